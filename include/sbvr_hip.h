@@ -1,0 +1,102 @@
+/*
+ * sbvr_hip.h -- C ABI of libsbvr_hip.so, the MI355X (gfx950) implementation of
+ * the SBVR compressed-domain linear layer.
+ *
+ * Every entry point takes plain device pointers and sizes, launches on the HIP
+ * stream it is given (a hipStream_t passed as void*; NULL is the default
+ * stream), never synchronises, never allocates and never throws: the return
+ * value is 0 on success or one of the negative SBVR_HIP_E* codes, and
+ * sbvr_hip_last_error() returns a text for the last failure on the calling
+ * thread.  Tensors are dense, row-major, in the layouts that sbvr/core.py of the
+ * reference produces (cited per function).
+ *
+ * The names below replace, one for one, the launchers that the reference's
+ * pybind wrappers call (sbvr/kernels/sbvr_ops.cpp); the file and lines of each
+ * are given with the declaration.
+ */
+#ifndef SBVR_HIP_H
+#define SBVR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SBVR_HIP_OK 0
+#define SBVR_HIP_EINVAL (-1)      /* null pointer, non-positive or misaligned size */
+#define SBVR_HIP_EUNSUPPORTED (-2) /* a shape or format no kernel here covers */
+#define SBVR_HIP_ELAUNCH (-3)     /* HIP reported an error at launch */
+#define SBVR_HIP_EWORKSPACE (-4)  /* workspace missing or too small */
+
+/* ABI version of this header (major*100 + minor). */
+int sbvr_hip_version(void);
+
+/* Text of the last error raised on this thread ("" if none). */
+const char *sbvr_hip_last_error(void);
+
+/* Checks that `device` is a gfx950 part and caches its properties.
+ * Replaces sbvr_cuda_init, sbvr/kernels/sbvr_ops.cpp:122-150. */
+int sbvr_hip_init(int device);
+
+/* Bytes of device workspace sbvr_hip_linear_f16 wants for this shape (0 if
+ * none).  The workspace must be zero-filled once after allocation; every call
+ * leaves it zero-filled where it needs zeros.  Calls that share a workspace
+ * must not overlap in time. */
+size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
+
+/*
+ * out[m,n] = f16( sum_g sum_j coeff_cache[coeff_idx[g,n], j]
+ *                   * sum_{k in group g, bit_j(n,k)=1} x[m,k] )  (+ bias[n])
+ *
+ * i.e. x @ decode(W)^T for a weight W (N,K) held in the reference's default
+ * layout (sbvr/core.py:724-731, 782-805):
+ *   x           (M, K)      fp16
+ *   bvr         (K/32, N, S) uint32, bit k%32 of bvr[k/32, n, j] = plane j of W[n,k]
+ *   coeff_idx   (K/G, N)    uint8 (idx_bytes 1) or uint16 (idx_bytes 2)
+ *   coeff_cache (L, S)      fp16
+ *   bias        (N) fp16 or NULL; added after the sum is rounded to fp16, as
+ *               sbvr/kernels/sbvr_kernel.cu:555-559 does
+ *   out         (M, N)      fp16
+ * fp32 accumulation, one rounding to fp16.  K must be a multiple of G and G of
+ * 32.  The reference has no kernel of exactly this form (its fp16-activation
+ * kernels, sbvr_kernel.cu:121-359 behind sbvr_ops.cpp:79-120, want the
+ * trans=True layout); this is the operator its models/sbvr_llama.py:86-87
+ * SBVRLinear.forward stands for.
+ * flags: bit 0 forces the portable kernel (one thread per output).
+ */
+int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_idx,
+                        int idx_bytes, const void *coeff_cache, const void *bias,
+                        void *out, int M, int N, int K, int S, int G, int L,
+                        void *workspace, size_t workspace_bytes, int flags,
+                        void *stream);
+
+/*
+ * fp16 activations against a weight encoded with trans=True (groups along N):
+ *   r_bvr (N/32, K, S) uint32, r_coeff_idx (N/G, K), r_coeff_cache (L, S) fp16
+ *   out[m,n] = f16( bias[n] + sum_k x[m,k] * sum_j c[idx[n/G,k], j] * bit_j )
+ * Replaces launch_cuda_sbvr_row_deq_mm_T, sbvr/kernels/sbvr_kernel.cu:876-912,
+ * called from sbvr_row_deq_mm_T, sbvr/kernels/sbvr_ops.cpp:79-120.
+ */
+int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_coeff_idx,
+                          int idx_bytes, const void *r_coeff_cache, const void *bias,
+                          void *out, int M, int N, int K, int S, int G, int L,
+                          void *stream);
+
+/*
+ * Both operands SBVR-encoded (default uint32 layout on both sides):
+ *   out[m,n] = f16( sum_g sum_l sum_r popcount_g(L_l & R_r) * a_l * b_r ) (+ bias[n])
+ * Replaces launch_cuda_sbvr_mm_T, sbvr/kernels/sbvr_kernel.cu:914-1022, called
+ * from sbvr_mm_T, sbvr/kernels/sbvr_ops.cpp:35-76.
+ */
+int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_bytes,
+                  const void *l_coeff_cache, const uint32_t *r_bvr,
+                  const void *r_coeff_idx, int r_idx_bytes, const void *r_coeff_cache,
+                  const void *bias, void *out, int M, int N, int K, int Sl, int Sr,
+                  int G, int Ll, int Lr, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SBVR_HIP_H */

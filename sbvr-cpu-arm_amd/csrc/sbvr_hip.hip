@@ -1,0 +1,747 @@
+// libsbvr_hip.so -- HIP kernels for gfx950 (MI355X) behind the C ABI of
+// include/sbvr_hip.h: the SBVR compressed-domain linear layer.
+//
+// Decode path (M <= 16), sbvr_gemv_mfma_kernel.  The work is one bit per weight
+// element and plane, far too many bits for one VALU lane-op each, so the masked
+// sums run on the matrix cores:
+//   * a 32-bit plane word becomes four dwords of fp4 (e2m1) values with one AND
+//     (or shift+AND) each: nibble q of dword t carries bit 4q+t of the word as
+//     0.5, 1.0 or 2.0;
+//   * the fp16 activations of one 128-element sub-group are written, once per
+//     workgroup, as three fp8 (e4m3) terms h1 + h2 + h3/256 = x * 2^e * f_t, which
+//     reproduce the fp16 value exactly (4 significant bits each, the third taken
+//     from the residual scaled by 256), in the register image of the A operand;
+//     the per-position factor f_t undoes the 0.5/1/2 of the B nibbles, 2^e is a
+//     power of two per (row, sub-group);
+//   * v_mfma_f32_16x16x128_f8f6f4 (A fp8, B fp4) then yields, for 16 columns
+//     and one plane, the three partial plane sums per batch row; they are added,
+//     rescaled and multiplied by the group's coefficient in fp32.
+// The packed layout of the reference (sbvr/core.py:724-731, 782-805) is read as
+// it is: a lane loads the S plane words of one (word, column) pair with one
+// vector load, 16 neighbouring columns give 256 contiguous bytes.
+//
+// Work split: a workgroup owns 64*CT columns and SP sub-groups of K; K is split
+// over workgroups, partial sums go to a workspace and the last workgroup to
+// finish a column tile adds them in a fixed order (deterministic result).
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../../include/sbvr_hip.h"
+
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+struct DevInfo {
+    bool ready = false;
+    int cus = 256;
+};
+DevInfo g_dev[16];
+
+// ------------------------------------------------------------------ helpers
+
+__device__ __forceinline__ float h2f(uint16_t h)
+{
+    return static_cast<float>(__builtin_bit_cast(_Float16, h));
+}
+
+__device__ __forceinline__ uint16_t f2h(float f)
+{
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+
+// fp16 add of two fp16 values: exact sum rounded once (what __hadd does).
+__device__ __forceinline__ uint16_t hadd(uint16_t a, uint16_t b)
+{
+    return f2h(h2f(a) + h2f(b));
+}
+
+template <typename IdxT>
+__device__ __forceinline__ int load_idx(const void *p, size_t i)
+{
+    return static_cast<int>(static_cast<const IdxT *>(p)[i]);
+}
+
+// ---------------------------------------------------- portable kernel (any shape)
+
+// One thread per output element.  Slow; used for shapes the MFMA kernel does
+// not take and as a second implementation to test against.
+template <typename IdxT>
+__global__ void __launch_bounds__(256)
+sbvr_linear_portable_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ bvr,
+                            const void *__restrict__ idx, const uint16_t *__restrict__ cache,
+                            const uint16_t *__restrict__ bias, uint16_t *__restrict__ out,
+                            int M, int N, int K, int S, int G)
+{
+    const size_t o = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (o >= static_cast<size_t>(M) * N)
+        return;
+    const int m = static_cast<int>(o / N), n = static_cast<int>(o % N);
+    const int wpg = G / 32;
+    float acc = 0.f;
+    for (int g = 0; g < K / G; ++g) {
+        const int line = load_idx<IdxT>(idx, static_cast<size_t>(g) * N + n);
+        for (int j = 0; j < S; ++j) {
+            float ps = 0.f;
+            for (int w = 0; w < wpg; ++w) {
+                const int kw = g * wpg + w;
+                uint32_t bits = bvr[(static_cast<size_t>(kw) * N + n) * S + j];
+                const uint16_t *xr = x + static_cast<size_t>(m) * K + kw * 32;
+                while (bits) {
+                    const int b = __builtin_ctz(bits);
+                    bits &= bits - 1;
+                    ps += h2f(xr[b]);
+                }
+            }
+            acc = fmaf(h2f(cache[static_cast<size_t>(line) * S + j]), ps, acc);
+        }
+    }
+    uint16_t r = f2h(acc);
+    if (bias)
+        r = hadd(r, bias[n]);
+    out[o] = r;
+}
+
+// --------------------------------------------------------------- MFMA decode
+
+constexpr int kSub = 128;        // K elements per MFMA (one sub-group)
+constexpr int kWavesPerWG = 4;
+constexpr int kThreads = 64 * kWavesPerWG;
+constexpr int kPipe = 8;         // units of weights in flight per wave
+constexpr int kMaxMT = 4;        // row tiles of 4 batch rows -> M <= 16
+constexpr float kLastTermScale = 256.f;  // third fp8 term of an activation holds residual * 256
+constexpr int kMaxTiles = 4096;  // column tiles of workgroups; fixes the counter area of the workspace
+constexpr size_t kCounterBytes = kMaxTiles * sizeof(unsigned);
+
+struct GemvArgs {
+    const uint16_t *x;
+    const uint32_t *bvr;
+    const void *idx;
+    const uint16_t *cache;
+    const uint16_t *bias;
+    uint16_t *out;
+    float *partial;       // (ksplit, M, N)
+    unsigned *counters;   // (n_tiles)
+    int M, N, K, G, L;
+    int CT;               // column tiles (16 columns) per wave
+    int SP;               // sub-groups per workgroup
+    int n_tiles;          // workgroups along N
+    int ksplit;           // workgroups along K
+};
+
+// Where element k (0..127) of row `row` (0..15) of a sub-group sits in the A
+// operand of v_mfma_f32_16x16x128_f8f6f4 with fp8 A and fp4 B, given that B
+// dword t, nibble q of the lane holding word c carries bit 4q+t of that word:
+//   B side: reduction index kk = 32c + 8t + q           (lane block c, nibble 8t+q)
+//   A side: byte p of lane 16*kb + row holds kk = 64*(p/16) + 16*kb + p%16
+__device__ __forceinline__ int a_image_byte_offset(int k, int row)
+{
+    const int c = k >> 5, r = k & 31, q = r >> 2, t = r & 3;
+    const int kk = 32 * c + 8 * t + q;
+    const int p = 16 * (kk >> 6) + (kk & 15);
+    const int lane = 16 * ((kk >> 4) & 3) + row;
+    return lane * 32 + p;
+}
+
+template <int S>
+struct Planes {
+    uint32_t w[S];
+};
+
+template <int S>
+__device__ __forceinline__ Planes<S> load_planes(const uint32_t *p)
+{
+    Planes<S> r;
+    if constexpr (S == 4) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p);
+        r.w[0] = v.x; r.w[1] = v.y; r.w[2] = v.z; r.w[3] = v.w;
+    } else if constexpr (S == 2) {
+        const uint2 v = *reinterpret_cast<const uint2 *>(p);
+        r.w[0] = v.x; r.w[1] = v.y;
+    } else if constexpr (S == 8) {
+        const uint4 v0 = reinterpret_cast<const uint4 *>(p)[0];
+        const uint4 v1 = reinterpret_cast<const uint4 *>(p)[1];
+        r.w[0] = v0.x; r.w[1] = v0.y; r.w[2] = v0.z; r.w[3] = v0.w;
+        r.w[4] = v1.x; r.w[5] = v1.y; r.w[6] = v1.z; r.w[7] = v1.w;
+    } else if constexpr (S == 6) {
+        const uint2 v0 = reinterpret_cast<const uint2 *>(p)[0];
+        const uint2 v1 = reinterpret_cast<const uint2 *>(p)[1];
+        const uint2 v2 = reinterpret_cast<const uint2 *>(p)[2];
+        r.w[0] = v0.x; r.w[1] = v0.y; r.w[2] = v1.x; r.w[3] = v1.y; r.w[4] = v2.x; r.w[5] = v2.y;
+    } else {
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+            r.w[j] = p[j];
+    }
+    return r;
+}
+
+// The S fp16 coefficients of one line, as floats.
+template <int S>
+__device__ __forceinline__ void load_coeffs(const uint16_t *cache, int line, float (&c)[S])
+{
+    const uint16_t *p = cache + static_cast<uint32_t>(line) * S;
+    if constexpr (S % 2 == 0) {
+        uint32_t v[S / 2];
+        if constexpr (S == 4) {
+            const uint2 t = *reinterpret_cast<const uint2 *>(p);
+            v[0] = t.x; v[1] = t.y;
+        } else if constexpr (S == 8) {
+            const uint4 t = *reinterpret_cast<const uint4 *>(p);
+            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < S / 2; ++j)
+                v[j] = reinterpret_cast<const uint32_t *>(p)[j];
+        }
+#pragma unroll
+        for (int j = 0; j < S / 2; ++j) {
+            c[2 * j] = h2f(static_cast<uint16_t>(v[j] & 0xffffu));
+            c[2 * j + 1] = h2f(static_cast<uint16_t>(v[j] >> 16));
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+            c[j] = h2f(p[j]);
+    }
+}
+
+template <int S, typename IdxT, int MT>
+__global__ void __launch_bounds__(kThreads)
+sbvr_gemv_mfma_kernel(const GemvArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    // smem: A images [SP][MT][64 lanes][32 bytes], then scales [SP][MT*4] floats
+    unsigned char *img = smem;
+    float *scales = reinterpret_cast<float *>(smem + static_cast<size_t>(a.SP) * MT * 2048);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int nt = blockIdx.x % a.n_tiles;
+    const int kp = blockIdx.x / a.n_tiles;
+    const int N = a.N, K = a.K;
+    const int col = lane & 15;   // column inside a tile (B and D operands)
+    const int blk = lane >> 4;   // word of the sub-group (B), batch row of the tile (D)
+    const int sg0 = kp * a.SP;   // first sub-group of this workgroup
+    const int gsub = a.G / kSub; // sub-groups per coefficient group
+    const int U = a.CT * a.SP;   // units (column tile x sub-group) of this wave
+    const int n_wave = (nt * kWavesPerWG + wave) * a.CT * 16;  // first column of this wave
+
+    // -- 1. start the weight stream: unit u = (column tile u / SP, sub-group u % SP)
+    Planes<S> q[kPipe];
+    int qline[kPipe];
+    int i_ct = 0, i_sg = 0;      // column tile and sub-group of the next unit to load
+    auto issue = [&](Planes<S> &dst, int &line) {
+        int n = n_wave + i_ct * 16 + col;
+        n = n < N ? n : N - 1;   // clamped lanes compute a value nobody stores
+        const uint32_t word = static_cast<uint32_t>(sg0 + i_sg) * 4 + blk;
+        dst = load_planes<S>(a.bvr + (word * N + n) * S);
+        line = load_idx<IdxT>(a.idx, static_cast<uint32_t>((sg0 + i_sg) / gsub) * N + n);
+        if (++i_sg == a.SP) {
+            i_sg = 0;
+            ++i_ct;
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < kPipe; ++i)
+        if (i < U)
+            issue(q[i], qline[i]);
+
+    // -- 2. A images of this workgroup's sub-groups
+    for (int i = tid; i < a.SP * MT * 512; i += kThreads)
+        reinterpret_cast<uint32_t *>(img)[i] = 0u;
+    __syncthreads();
+    for (int task = wave; task < a.SP * a.M; task += kWavesPerWG) {
+        const int sgi = task / a.M, m = task - sgi * a.M;
+        const uint32_t xx = *reinterpret_cast<const uint32_t *>(
+            a.x + static_cast<size_t>(m) * K + static_cast<size_t>(sg0 + sgi) * kSub + 2 * lane);
+        const float x0 = h2f(static_cast<uint16_t>(xx & 0xffffu));
+        const float x1 = h2f(static_cast<uint16_t>(xx >> 16));
+        float amax = fmaxf(fabsf(x0), fabsf(x1));
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+            amax = fmaxf(amax, __shfl_xor(amax, o));
+        // 2^e puts the largest magnitude into [32, 64)
+        const int E = static_cast<int>((__float_as_uint(amax) >> 23) & 255u) - 127;
+        const int e = (amax > 0.f && E < 100) ? 5 - E : 0;
+        const float up = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+        const int mt = m >> 2, row = (m & 3) * 4;
+        unsigned char *dst = img + static_cast<size_t>(sgi * MT + mt) * 2048;
+        if (lane == 0)   // products come out as 2*x*2^e
+            scales[sgi * (MT * 4) + m] = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k = 2 * lane + h;
+            const int t = k & 3;
+            float z = (h ? x1 : x0) * up * (t == 0 ? 4.f : (t == 1 ? 2.f : 1.f));
+            // h1 + h2 + h3/256 == z exactly: each fp8 takes the next 4 significant
+            // bits, the last one of the residual scaled up out of the subnormals
+#pragma unroll
+            for (int term = 0; term < 3; ++term) {
+                if (term == 2)
+                    z *= kLastTermScale;
+                const int b = __builtin_amdgcn_cvt_pk_fp8_f32(z, 0.f, 0, false) & 0xff;
+                z -= __builtin_amdgcn_cvt_f32_fp8(b, 0);
+                dst[a_image_byte_offset(k, row + term)] = static_cast<unsigned char>(b);
+            }
+        }
+    }
+    __syncthreads();
+
+    // -- 3. stream the units
+    float y[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+        y[i] = 0.f;
+
+    auto finish_tile = [&](int ct) {
+        const int n = n_wave + ct * 16 + col;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 4 + blk;
+            if (n < N && m < a.M) {
+                if (a.ksplit == 1) {
+                    uint16_t r = f2h(y[mt]);
+                    if (a.bias)
+                        r = hadd(r, a.bias[n]);
+                    a.out[static_cast<size_t>(m) * N + n] = r;
+                } else {
+                    a.partial[(static_cast<size_t>(kp) * a.M + m) * N + n] = y[mt];
+                }
+            }
+            y[mt] = 0.f;
+        }
+    };
+
+    int p_ct = 0, p_sg = 0;      // column tile and sub-group of the unit being processed
+    auto process = [&](const Planes<S> &pl, int line) {
+        const int ct = p_ct, sgi = p_sg;
+        float c[S];
+        load_coeffs<S>(a.cache, min(line, a.L - 1), c);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const v8i A = *reinterpret_cast<const v8i *>(img + static_cast<size_t>(sgi * MT + mt) * 2048 + lane * 32);
+            const float sc = scales[sgi * (MT * 4) + mt * 4 + blk];
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < S; ++j) {
+                const uint32_t w = pl.w[j];
+                v8i B;
+                B[0] = static_cast<int>(w & 0x11111111u);
+                B[1] = static_cast<int>(w & 0x22222222u);
+                B[2] = static_cast<int>(w & 0x44444444u);
+                B[3] = static_cast<int>((w >> 1) & 0x44444444u);
+                B[4] = 0; B[5] = 0; B[6] = 0; B[7] = 0;
+                const v4f z = {0.f, 0.f, 0.f, 0.f};
+                const v4f D = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, z, 0, 4, 0, 0, 0, 0);
+                acc = fmaf(c[j], fmaf(D[2], 1.f / kLastTermScale, D[0] + D[1]), acc);
+            }
+            y[mt] = fmaf(acc, sc, y[mt]);
+        }
+        if (++p_sg == a.SP) {
+            p_sg = 0;
+            ++p_ct;
+            finish_tile(ct);
+        }
+    };
+
+    for (int u0 = 0; u0 < U; u0 += kPipe) {
+#pragma unroll
+        for (int i = 0; i < kPipe; ++i) {
+            const int u = u0 + i;
+            if (u < U) {
+                const Planes<S> pl = q[i];
+                const int line = qline[i];
+                if (u + kPipe < U)
+                    issue(q[i], qline[i]);
+                process(pl, line);
+            }
+        }
+    }
+
+    // -- 4. split K: the last workgroup of a column tile adds the partial sums
+    if (a.ksplit > 1) {
+        __shared__ int s_last;
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned prev = atomicAdd(&a.counters[nt], 1u);
+            s_last = (prev == static_cast<unsigned>(a.ksplit - 1));
+        }
+        __syncthreads();
+        if (s_last) {
+            __threadfence();
+            const int cols = kWavesPerWG * a.CT * 16;
+            const int n0 = nt * cols;
+            for (int i = tid; i < cols * a.M; i += kThreads) {
+                const int m = i / cols, n = n0 + (i - m * cols);
+                if (n < N) {
+                    float s = 0.f;
+                    for (int p = 0; p < a.ksplit; ++p)
+                        s += a.partial[(static_cast<size_t>(p) * a.M + m) * N + n];
+                    uint16_t r = f2h(s);
+                    if (a.bias)
+                        r = hadd(r, a.bias[n]);
+                    a.out[static_cast<size_t>(m) * N + n] = r;
+                }
+            }
+            if (tid == 0)
+                a.counters[nt] = 0u;
+        }
+    }
+}
+
+// Launch shape for the MFMA kernel.
+struct GemvPlan {
+    int CT, SP, n_tiles, ksplit, MT;
+    size_t lds;
+};
+
+int env_int(const char *name, int dflt)
+{
+    const char *v = getenv(name);
+    return v && *v ? atoi(v) : dflt;
+}
+
+GemvPlan plan_gemv(int M, int N, int K, int cus)
+{
+    const int nsub = K / kSub;
+    const int MT = (M + 3) / 4;
+    const int tiles16 = (N + 15) / 16;
+    GemvPlan best{};
+    double best_cost = 1e30;
+    for (int SP = 1; SP <= nsub && SP <= 8; ++SP) {
+        if (nsub % SP)
+            continue;
+        for (int CT = 1; CT <= 8; ++CT) {
+            const int U = CT * SP;
+            if (U > 16)
+                continue;
+            const int n_tiles = (tiles16 + kWavesPerWG * CT - 1) / (kWavesPerWG * CT);
+            const int ksplit = nsub / SP;
+            const long wgs = static_cast<long>(n_tiles) * ksplit;
+            // two workgroups per CU run at once; every workgroup pays a fixed
+            // start-up (about 6 units' worth) and its share of the A images
+            const double rounds = static_cast<double>((wgs + 2L * cus - 1) / (2L * cus));
+            const double per_wg = U + 6.0 + 0.5 * SP * M;
+            const double waste = static_cast<double>(n_tiles) * kWavesPerWG * CT / tiles16;
+            const double cost = rounds * per_wg * waste + 0.02 * ksplit;
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = GemvPlan{CT, SP, n_tiles, ksplit, MT, 0};
+            }
+        }
+    }
+    const int eCT = env_int("SBVR_HIP_CT", 0), eSP = env_int("SBVR_HIP_SP", 0);
+    if (eCT > 0 && eSP > 0 && nsub % eSP == 0) {
+        best.CT = eCT;
+        best.SP = eSP;
+        best.n_tiles = (tiles16 + kWavesPerWG * eCT - 1) / (kWavesPerWG * eCT);
+        best.ksplit = nsub / eSP;
+    }
+    best.MT = MT;
+    best.lds = static_cast<size_t>(best.SP) * MT * 2048 + static_cast<size_t>(best.SP) * MT * 4 * sizeof(float);
+    return best;
+}
+
+bool mfma_path_ok(int M, int N, int K, int S, int G)
+{
+    // 32-bit element offsets into bvr; one counter per workgroup column tile
+    return M >= 1 && M <= 4 * kMaxMT && K % kSub == 0 && G % kSub == 0 &&
+           (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) &&
+           static_cast<double>(K / 32) * N * S < 2147483648.0 && (N + 63) / 64 <= kMaxTiles;
+}
+
+template <int S, typename IdxT>
+hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
+{
+    const dim3 grid(static_cast<unsigned>(p.n_tiles) * p.ksplit), block(kThreads);
+    switch (p.MT) {
+    case 1: hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, IdxT, 1>), grid, block, p.lds, st, a); break;
+    case 2: hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, IdxT, 2>), grid, block, p.lds, st, a); break;
+    case 3: hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, IdxT, 3>), grid, block, p.lds, st, a); break;
+    default: hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, IdxT, 4>), grid, block, p.lds, st, a); break;
+    }
+    return hipGetLastError();
+}
+
+template <typename IdxT>
+hipError_t launch_gemv_s(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t st)
+{
+    switch (S) {
+    case 2: return launch_gemv_mt<2, IdxT>(a, p, st);
+    case 3: return launch_gemv_mt<3, IdxT>(a, p, st);
+    case 4: return launch_gemv_mt<4, IdxT>(a, p, st);
+    case 6: return launch_gemv_mt<6, IdxT>(a, p, st);
+    default: return launch_gemv_mt<8, IdxT>(a, p, st);
+    }
+}
+
+int current_cus()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
+        return 256;
+    if (!g_dev[dev].ready) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
+            g_dev[dev].cus = prop.multiProcessorCount;
+            g_dev[dev].ready = true;
+        }
+    }
+    return g_dev[dev].cus;
+}
+
+// -------------------------------------------- trans=True and both-encoded forms
+
+// One thread per output; the lanes of a wave share k and differ in n, so the
+// plane words and indices are wave-uniform broadcasts.
+template <typename IdxT>
+__global__ void __launch_bounds__(256)
+sbvr_row_deq_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ bvr,
+                    const void *__restrict__ idx, const uint16_t *__restrict__ cache,
+                    const uint16_t *__restrict__ bias, uint16_t *__restrict__ out,
+                    int M, int N, int K, int S, int G)
+{
+    const size_t o = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (o >= static_cast<size_t>(M) * N)
+        return;
+    const int m = static_cast<int>(o / N), n = static_cast<int>(o % N);
+    float acc = bias ? h2f(bias[n]) : 0.f;
+    for (int k = 0; k < K; ++k) {
+        const int line = load_idx<IdxT>(idx, static_cast<size_t>(n / G) * K + k);
+        float w = 0.f;
+        for (int j = 0; j < S; ++j) {
+            const uint32_t bits = bvr[(static_cast<size_t>(n >> 5) * K + k) * S + j];
+            if ((bits >> (n & 31)) & 1u)
+                w += h2f(cache[static_cast<size_t>(line) * S + j]);
+        }
+        acc = fmaf(h2f(x[static_cast<size_t>(m) * K + k]), w, acc);
+    }
+    out[o] = f2h(acc);
+}
+
+template <typename LIdxT, typename RIdxT>
+__global__ void __launch_bounds__(256)
+sbvr_mm_T_kernel(const uint32_t *__restrict__ l_bvr, const void *__restrict__ l_idx,
+                 const uint16_t *__restrict__ l_cache, const uint32_t *__restrict__ r_bvr,
+                 const void *__restrict__ r_idx, const uint16_t *__restrict__ r_cache,
+                 const uint16_t *__restrict__ bias, uint16_t *__restrict__ out,
+                 int M, int N, int K, int Sl, int Sr, int G)
+{
+    const size_t o = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (o >= static_cast<size_t>(M) * N)
+        return;
+    const int m = static_cast<int>(o / N), n = static_cast<int>(o % N);
+    const int wpg = G / 32;
+    float acc = 0.f;
+    for (int g = 0; g < K / G; ++g) {
+        const uint16_t *ca = l_cache + static_cast<size_t>(load_idx<LIdxT>(l_idx, static_cast<size_t>(g) * M + m)) * Sl;
+        const uint16_t *cb = r_cache + static_cast<size_t>(load_idx<RIdxT>(r_idx, static_cast<size_t>(g) * N + n)) * Sr;
+        for (int l = 0; l < Sl; ++l) {
+            const float al = h2f(ca[l]);
+            for (int r = 0; r < Sr; ++r) {
+                int pc = 0;
+                for (int w = 0; w < wpg; ++w) {
+                    const size_t kw = static_cast<size_t>(g) * wpg + w;
+                    pc += __builtin_popcount(l_bvr[(kw * M + m) * Sl + l] & r_bvr[(kw * N + n) * Sr + r]);
+                }
+                acc = fmaf(static_cast<float>(pc), al * h2f(cb[r]), acc);
+            }
+        }
+    }
+    uint16_t res = f2h(acc);
+    if (bias)
+        res = hadd(res, bias[n]);
+    out[o] = res;
+}
+
+} // namespace
+
+// ------------------------------------------------------------------- C ABI
+
+extern "C" {
+
+int sbvr_hip_version(void) { return 100; }
+
+const char *sbvr_hip_last_error(void) { return g_err; }
+
+int sbvr_hip_init(int device)
+{
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(SBVR_HIP_ELAUNCH, "no HIP device: %s", hipGetErrorString(e));
+    if (device < 0 || device >= count || device >= 16)
+        return fail(SBVR_HIP_EINVAL, "device %d out of range (%d devices)", device, count);
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess)
+        return fail(SBVR_HIP_ELAUNCH, "hipGetDeviceProperties: %s", hipGetErrorString(e));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(SBVR_HIP_EUNSUPPORTED, "device %d is %s; this library is built for gfx950 only",
+                    device, prop.gcnArchName);
+    g_dev[device].cus = prop.multiProcessorCount;
+    g_dev[device].ready = true;
+    return SBVR_HIP_OK;
+}
+
+size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G)
+{
+    if (!mfma_path_ok(M, N, K, S, G))
+        return 0;
+    // the plan depends on the CU count; size for the worst case over plans:
+    // the counter area + ksplit*M*N floats with ksplit <= K/128
+    return kCounterBytes + static_cast<size_t>(K / kSub) * M * N * sizeof(float);
+}
+
+int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_idx,
+                        int idx_bytes, const void *coeff_cache, const void *bias,
+                        void *out, int M, int N, int K, int S, int G, int L,
+                        void *workspace, size_t workspace_bytes, int flags,
+                        void *stream)
+{
+    if (!x || !bvr || !coeff_idx || !coeff_cache || !out)
+        return fail(SBVR_HIP_EINVAL, "null pointer argument");
+    if (M <= 0 || N <= 0 || K <= 0 || S <= 0 || G <= 0 || L <= 0)
+        return fail(SBVR_HIP_EINVAL, "non-positive size (M=%d N=%d K=%d S=%d G=%d L=%d)", M, N, K, S, G, L);
+    if (G % 32 != 0 || K % G != 0)
+        return fail(SBVR_HIP_EINVAL, "K=%d must be a multiple of G=%d, and G of 32", K, G);
+    if (idx_bytes != 1 && idx_bytes != 2)
+        return fail(SBVR_HIP_EINVAL, "idx_bytes must be 1 or 2, got %d", idx_bytes);
+    if (idx_bytes == 1 && L > 256)
+        return fail(SBVR_HIP_EINVAL, "uint8 indices cannot address L=%d lines", L);
+    if (static_cast<size_t>(M) * N > 0x7fffffffu)
+        return fail(SBVR_HIP_EUNSUPPORTED, "M*N too large");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    const bool aligned = reinterpret_cast<uintptr_t>(bvr) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&
+                         reinterpret_cast<uintptr_t>(coeff_cache) % 16 == 0;
+    if (!(flags & 1) && aligned && mfma_path_ok(M, N, K, S, G)) {
+        const GemvPlan p = plan_gemv(M, N, K, current_cus());
+        GemvArgs a{};
+        a.x = static_cast<const uint16_t *>(x);
+        a.bvr = bvr;
+        a.idx = coeff_idx;
+        a.cache = static_cast<const uint16_t *>(coeff_cache);
+        a.bias = static_cast<const uint16_t *>(bias);
+        a.out = static_cast<uint16_t *>(out);
+        a.M = M; a.N = N; a.K = K; a.G = G; a.L = L;
+        a.CT = p.CT; a.SP = p.SP; a.n_tiles = p.n_tiles; a.ksplit = p.ksplit;
+        if (p.ksplit > 1) {
+            const size_t counters = kCounterBytes;
+            const size_t need = counters + static_cast<size_t>(p.ksplit) * M * N * sizeof(float);
+            if (!workspace || workspace_bytes < need)
+                return fail(SBVR_HIP_EWORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+            a.counters = static_cast<unsigned *>(workspace);
+            a.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + counters);
+        }
+        const hipError_t e = (idx_bytes == 1) ? launch_gemv_s<uint8_t>(S, a, p, st) : launch_gemv_s<uint16_t>(S, a, p, st);
+        if (e != hipSuccess)
+            return fail(SBVR_HIP_ELAUNCH, "gemv launch: %s", hipGetErrorString(e));
+        return SBVR_HIP_OK;
+    }
+
+    const size_t total = static_cast<size_t>(M) * N;
+    const dim3 grid(static_cast<unsigned>((total + 255) / 256)), block(256);
+    if (idx_bytes == 1)
+        hipLaunchKernelGGL(sbvr_linear_portable_kernel<uint8_t>, grid, block, 0, st,
+                           static_cast<const uint16_t *>(x), bvr, coeff_idx, static_cast<const uint16_t *>(coeff_cache),
+                           static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out), M, N, K, S, G);
+    else
+        hipLaunchKernelGGL(sbvr_linear_portable_kernel<uint16_t>, grid, block, 0, st,
+                           static_cast<const uint16_t *>(x), bvr, coeff_idx, static_cast<const uint16_t *>(coeff_cache),
+                           static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out), M, N, K, S, G);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return fail(SBVR_HIP_ELAUNCH, "portable launch: %s", hipGetErrorString(e));
+    return SBVR_HIP_OK;
+}
+
+int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_coeff_idx,
+                          int idx_bytes, const void *r_coeff_cache, const void *bias,
+                          void *out, int M, int N, int K, int S, int G, int L,
+                          void *stream)
+{
+    if (!x || !r_bvr || !r_coeff_idx || !r_coeff_cache || !out)
+        return fail(SBVR_HIP_EINVAL, "null pointer argument");
+    if (M <= 0 || N <= 0 || K <= 0 || S <= 0 || G <= 0 || L <= 0)
+        return fail(SBVR_HIP_EINVAL, "non-positive size");
+    if (N % 32 != 0 || G % 32 != 0 || N % G != 0)
+        return fail(SBVR_HIP_EINVAL, "N=%d must be a multiple of G=%d, and G of 32", N, G);
+    if (idx_bytes != 1 && idx_bytes != 2)
+        return fail(SBVR_HIP_EINVAL, "idx_bytes must be 1 or 2, got %d", idx_bytes);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t total = static_cast<size_t>(M) * N;
+    const dim3 grid(static_cast<unsigned>((total + 255) / 256)), block(256);
+    if (idx_bytes == 1)
+        hipLaunchKernelGGL(sbvr_row_deq_kernel<uint8_t>, grid, block, 0, st,
+                           static_cast<const uint16_t *>(x), r_bvr, r_coeff_idx, static_cast<const uint16_t *>(r_coeff_cache),
+                           static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out), M, N, K, S, G);
+    else
+        hipLaunchKernelGGL(sbvr_row_deq_kernel<uint16_t>, grid, block, 0, st,
+                           static_cast<const uint16_t *>(x), r_bvr, r_coeff_idx, static_cast<const uint16_t *>(r_coeff_cache),
+                           static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out), M, N, K, S, G);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return fail(SBVR_HIP_ELAUNCH, "row_deq launch: %s", hipGetErrorString(e));
+    return SBVR_HIP_OK;
+}
+
+int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_bytes,
+                  const void *l_coeff_cache, const uint32_t *r_bvr,
+                  const void *r_coeff_idx, int r_idx_bytes, const void *r_coeff_cache,
+                  const void *bias, void *out, int M, int N, int K, int Sl, int Sr,
+                  int G, int Ll, int Lr, void *stream)
+{
+    if (!l_bvr || !l_coeff_idx || !l_coeff_cache || !r_bvr || !r_coeff_idx || !r_coeff_cache || !out)
+        return fail(SBVR_HIP_EINVAL, "null pointer argument");
+    if (M <= 0 || N <= 0 || K <= 0 || Sl <= 0 || Sr <= 0 || G <= 0 || Ll <= 0 || Lr <= 0)
+        return fail(SBVR_HIP_EINVAL, "non-positive size");
+    if (G % 32 != 0 || K % G != 0)
+        return fail(SBVR_HIP_EINVAL, "K=%d must be a multiple of G=%d, and G of 32", K, G);
+    if ((l_idx_bytes != 1 && l_idx_bytes != 2) || (r_idx_bytes != 1 && r_idx_bytes != 2))
+        return fail(SBVR_HIP_EINVAL, "idx_bytes must be 1 or 2");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t total = static_cast<size_t>(M) * N;
+    const dim3 grid(static_cast<unsigned>((total + 255) / 256)), block(256);
+    const uint16_t *lc = static_cast<const uint16_t *>(l_coeff_cache), *rc = static_cast<const uint16_t *>(r_coeff_cache);
+    const uint16_t *b = static_cast<const uint16_t *>(bias);
+    uint16_t *o = static_cast<uint16_t *>(out);
+#define SBVR_MM_LAUNCH(LT, RT)                                                                   \
+    hipLaunchKernelGGL((sbvr_mm_T_kernel<LT, RT>), grid, block, 0, st, l_bvr, l_coeff_idx, lc,   \
+                       r_bvr, r_coeff_idx, rc, b, o, M, N, K, Sl, Sr, G)
+    if (l_idx_bytes == 1 && r_idx_bytes == 1)
+        SBVR_MM_LAUNCH(uint8_t, uint8_t);
+    else if (l_idx_bytes == 1)
+        SBVR_MM_LAUNCH(uint8_t, uint16_t);
+    else if (r_idx_bytes == 1)
+        SBVR_MM_LAUNCH(uint16_t, uint8_t);
+    else
+        SBVR_MM_LAUNCH(uint16_t, uint16_t);
+#undef SBVR_MM_LAUNCH
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return fail(SBVR_HIP_ELAUNCH, "mm_T launch: %s", hipGetErrorString(e));
+    return SBVR_HIP_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,202 @@
+"""Python binding of libsbvr_hip.so (ctypes over the C ABI of include/sbvr_hip.h).
+
+The functions keep the names, argument order and conventions of the reference's
+pybind operators (sbvr/kernels/sbvr_ops.cpp:152-172): sizes are taken from the
+tensor shapes, the output is allocated here, "no bias" is a 0-length tensor.
+Unlike the reference they check dtype, device and contiguity, and launch on
+torch's current HIP stream.  There is no CPU fallback: a missing library or a
+tensor that is not on a GPU raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_LIB_NAME = "libsbvr_hip.so"
+_lib = None
+_workspaces = {}
+
+
+class SbvrHipError(RuntimeError):
+    pass
+
+
+def library_path():
+    here = os.path.dirname(os.path.abspath(__file__))
+    return os.path.join(os.path.dirname(here), "csrc", _LIB_NAME)
+
+
+def _load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise SbvrHipError(f"{path} is missing: build it with `make -C {os.path.dirname(path)}` "
+                           "(or __graft_entry__.build()); there is no fallback path")
+    lib = ctypes.CDLL(path)
+    vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    lib.sbvr_hip_version.restype = i
+    lib.sbvr_hip_last_error.restype = ctypes.c_char_p
+    lib.sbvr_hip_init.argtypes = [i]
+    lib.sbvr_hip_linear_f16_workspace.restype = sz
+    lib.sbvr_hip_linear_f16_workspace.argtypes = [i, i, i, i, i]
+    lib.sbvr_hip_linear_f16.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp, sz, i, vp]
+    lib.sbvr_hip_row_deq_mm_T.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp]
+    lib.sbvr_hip_mm_T.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
+    _lib = lib
+    return lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise SbvrHipError(f"libsbvr_hip: error {rc}: {_load().sbvr_hip_last_error().decode()}")
+
+
+def _sbvr_hip_init(device=None):
+    """Counterpart of ``_sbvr_cuda_init`` (sbvr_ops.cpp:122-150): verifies the
+    device is a gfx950 part."""
+    dev = torch.cuda.current_device() if device is None else torch.device(device).index or 0
+    _check(_load().sbvr_hip_init(int(dev)))
+
+
+_sbvr_cuda_init = _sbvr_hip_init
+
+
+def _want(t, name, dtype=None, dim=None, device=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a tensor")
+    if not t.is_cuda:
+        raise SbvrHipError(f"{name} must be on a GPU (got {t.device}); this package has no CPU path")
+    if device is not None and t.device != device:
+        raise SbvrHipError(f"{name} is on {t.device}, expected {device}")
+    if dtype is not None and t.dtype not in (dtype if isinstance(dtype, tuple) else (dtype,)):
+        raise TypeError(f"{name} must have dtype {dtype}, got {t.dtype}")
+    if dim is not None and t.dim() != dim:
+        raise ValueError(f"{name} must have {dim} dimensions, got shape {tuple(t.shape)}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return t
+
+
+def _idx_bytes(idx, lines, name):
+    want = torch.uint8 if lines <= 256 else torch.uint16      # sbvr_kernel.cu:931-932
+    if idx.dtype != want:
+        raise TypeError(f"{name} must be {want} for {lines} coefficient lines, got {idx.dtype}")
+    return idx.element_size()
+
+
+def _bias_ptr(bias, n, device):
+    """Bias is used only when its length is N (sbvr_ops.cpp:56-58)."""
+    if bias is None or bias.numel() == 0 or bias.size(0) != n:
+        return None
+    _want(bias, "bias", torch.float16, 1, device)
+    return bias.data_ptr()
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _workspace(nbytes, device):
+    """Zero-initialised scratch per (device, stream); grown on demand.  The
+    kernels leave the part that must be zero zeroed."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _sbvr_linear_f16(x, bvr, coeff_idx, coeff_cache, bias=None, bvr_len=None, out=None, flags=0):
+    """y = x @ decode(W)^T (+ bias) for fp16 ``x`` (M, K) and a weight in the
+    default uint32 layout: ``bvr`` (K/32, N, S), ``coeff_idx`` (K/G, N),
+    ``coeff_cache`` (L, S).  Returns fp16 (M, N)."""
+    lib = _load()
+    dev = x.device
+    _want(x, "x", torch.float16, 2)
+    _want(bvr, "bvr", torch.uint32, 3, dev)
+    _want(coeff_idx, "coeff_idx", (torch.uint8, torch.uint16), 2, dev)
+    _want(coeff_cache, "coeff_cache", torch.float16, 2, dev)
+    M, K = x.shape
+    Kw, N, S = bvr.shape
+    L = coeff_cache.shape[0]
+    if Kw * 32 != K:
+        raise ValueError(f"x has K={K} but bvr holds {Kw * 32} columns")
+    if coeff_idx.shape[1] != N or coeff_cache.shape[1] != S:
+        raise ValueError("coeff_idx / coeff_cache shapes do not match bvr")
+    G = bvr_len if bvr_len is not None else K // coeff_idx.shape[0]
+    if G * coeff_idx.shape[0] != K:
+        raise ValueError(f"coeff_idx has {coeff_idx.shape[0]} groups, K={K}, bvr_len={G}")
+    ib = _idx_bytes(coeff_idx, L, "coeff_idx")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    else:
+        _want(out, "out", torch.float16, 2, dev)
+        if tuple(out.shape) != (M, N):
+            raise ValueError("out has the wrong shape")
+    need = lib.sbvr_hip_linear_f16_workspace(M, N, K, S, G)
+    ws = _workspace(need, dev) if need else None
+    with torch.cuda.device(dev):
+        _check(lib.sbvr_hip_linear_f16(
+            x.data_ptr(), bvr.data_ptr(), coeff_idx.data_ptr(), ib, coeff_cache.data_ptr(),
+            _bias_ptr(bias, N, dev), out.data_ptr(), M, N, K, S, G, L,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            int(flags), _stream()))
+    return out
+
+
+def _sbvr_row_deq_mm_T(l_w, r_bvr, r_coeff_idx, r_coeff_cache, bias, use_shfl=0, bvr_len=None):
+    """fp16 ``l_w`` (M, K) against a ``trans=True`` weight: ``r_bvr`` (N/32, K, S),
+    ``r_coeff_idx`` (N/G, K) (sbvr_ops.cpp:79-120).  ``use_shfl`` selected between
+    equivalent CUDA kernels in the reference and is ignored."""
+    lib = _load()
+    dev = l_w.device
+    _want(l_w, "l_w", torch.float16, 2)
+    _want(r_bvr, "r_bvr", torch.uint32, 3, dev)
+    _want(r_coeff_idx, "r_coeff_idx", (torch.uint8, torch.uint16), 2, dev)
+    _want(r_coeff_cache, "r_coeff_cache", torch.float16, 2, dev)
+    M, K = l_w.shape
+    Nw, K2, S = r_bvr.shape
+    N = Nw * 32
+    L = r_coeff_cache.shape[0]
+    if K2 != K or r_coeff_idx.shape[1] != K or r_coeff_cache.shape[1] != S:
+        raise ValueError("operand shapes do not match")
+    G = bvr_len if bvr_len is not None else N // r_coeff_idx.shape[0]
+    ib = _idx_bytes(r_coeff_idx, L, "r_coeff_idx")
+    out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.sbvr_hip_row_deq_mm_T(l_w.data_ptr(), r_bvr.data_ptr(), r_coeff_idx.data_ptr(), ib,
+                                         r_coeff_cache.data_ptr(), _bias_ptr(bias, N, dev), out.data_ptr(),
+                                         M, N, K, S, G, L, _stream()))
+    return out
+
+
+def _sbvr_mm_T(l_bvr, l_coeff_idx, l_coeff_cache, r_bvr, r_coeff_idx, r_coeff_cache, bias, bvr_len=None):
+    """Both operands encoded, default uint32 layout: ``l_bvr`` (K/32, M, Sl),
+    ``r_bvr`` (K/32, N, Sr) (sbvr_ops.cpp:35-76).  Returns fp16 (M, N)."""
+    lib = _load()
+    dev = l_bvr.device
+    _want(l_bvr, "l_bvr", torch.uint32, 3)
+    _want(r_bvr, "r_bvr", torch.uint32, 3, dev)
+    _want(l_coeff_idx, "l_coeff_idx", (torch.uint8, torch.uint16), 2, dev)
+    _want(r_coeff_idx, "r_coeff_idx", (torch.uint8, torch.uint16), 2, dev)
+    _want(l_coeff_cache, "l_coeff_cache", torch.float16, 2, dev)
+    _want(r_coeff_cache, "r_coeff_cache", torch.float16, 2, dev)
+    Kw, M, Sl = l_bvr.shape
+    Kw2, N, Sr = r_bvr.shape
+    if Kw != Kw2:
+        raise ValueError(f"operands disagree on K: {Kw * 32} vs {Kw2 * 32}")
+    K = Kw * 32
+    G = bvr_len if bvr_len is not None else K // l_coeff_idx.shape[0]
+    if l_coeff_idx.shape != (K // G, M) or r_coeff_idx.shape != (K // G, N):
+        raise ValueError("coeff_idx shapes do not match the operands")
+    Ll, Lr = l_coeff_cache.shape[0], r_coeff_cache.shape[0]
+    out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.sbvr_hip_mm_T(l_bvr.data_ptr(), l_coeff_idx.data_ptr(), _idx_bytes(l_coeff_idx, Ll, "l_coeff_idx"),
+                                 l_coeff_cache.data_ptr(), r_bvr.data_ptr(), r_coeff_idx.data_ptr(),
+                                 _idx_bytes(r_coeff_idx, Lr, "r_coeff_idx"), r_coeff_cache.data_ptr(),
+                                 _bias_ptr(bias, N, dev), out.data_ptr(), M, N, K, Sl, Sr, G, Ll, Lr, _stream()))
+    return out
