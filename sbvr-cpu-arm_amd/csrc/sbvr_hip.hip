@@ -124,11 +124,19 @@ sbvr_linear_portable_kernel(const uint16_t *__restrict__ x, const uint32_t *__re
 constexpr int kSub = 128;        // K elements per MFMA (one sub-group)
 constexpr int kWavesPerWG = 4;
 constexpr int kThreads = 64 * kWavesPerWG;
-constexpr int kPipe = 8;         // units of weights in flight per wave
-constexpr int kMaxMT = 4;        // row tiles of 4 batch rows -> M <= 16
+constexpr int kMaxM = 16;        // batch rows of the decode kernel (row tiles of 4)
 constexpr float kLastTermScale = 256.f;  // third fp8 term of an activation holds residual * 256
-constexpr int kMaxTiles = 4096;  // column tiles of workgroups; fixes the counter area of the workspace
-constexpr size_t kCounterBytes = kMaxTiles * sizeof(unsigned);
+constexpr int kTableRegs = 4;             // uint4 per thread while the coefficient table is staged
+constexpr size_t kMaxTableLds = kTableRegs * 16 * 256;   // largest coefficient table staged in LDS (16 KB)
+
+// Split-K accumulator: one 64-bit word per output, [count:8 | sum:56].  Every
+// workgroup adds (1 << 56) + (v + 2^47) with v = rint(partial * 2^30); integer
+// addition is exact and order-free, so the result does not depend on which
+// workgroup comes first.  The adder that finds count == ksplit-1 owns the total.
+constexpr int kAccFracBits = 30;
+constexpr long long kAccBias = 1ll << 47;
+constexpr float kAccClamp = 130000.f;    // |partial| beyond this becomes +-inf in fp16 anyway
+constexpr int kMaxKsplit = 255;
 
 struct GemvArgs {
     const uint16_t *x;
@@ -137,14 +145,16 @@ struct GemvArgs {
     const uint16_t *cache;
     const uint16_t *bias;
     uint16_t *out;
-    float *partial;       // (ksplit, M, N)
-    unsigned *counters;   // (n_tiles)
+    unsigned long long *acc;   // (M, N) split-K accumulators, all zero between calls
     int M, N, K, G, L;
-    int CT;               // column tiles (16 columns) per wave
-    int SP;               // sub-groups per workgroup
+    int idx16;            // coeff_idx holds uint16 (else uint8)
     int n_tiles;          // workgroups along N
     int ksplit;           // workgroups along K
+    int table_in_lds;     // coefficient table copied to LDS
+    int dbg;
 };
+
+__host__ __device__ constexpr size_t align16(size_t v) { return (v + 15) & ~static_cast<size_t>(15); }
 
 // Where element k (0..127) of row `row` (0..15) of a sub-group sits in the A
 // operand of v_mfma_f32_16x16x128_f8f6f4 with fp8 A and fp4 B, given that B
@@ -193,11 +203,11 @@ __device__ __forceinline__ Planes<S> load_planes(const uint32_t *p)
     return r;
 }
 
-// The S fp16 coefficients of one line, as floats.
-template <int S>
-__device__ __forceinline__ void load_coeffs(const uint16_t *cache, int line, float (&c)[S])
+// The S fp16 coefficients of one line, as floats.  P is an LDS or a global pointer.
+template <int S, typename P>
+__device__ __forceinline__ void load_coeffs(P cache, int line, float (&c)[S])
 {
-    const uint16_t *p = cache + static_cast<uint32_t>(line) * S;
+    P p = cache + static_cast<uint32_t>(line) * S;
     if constexpr (S % 2 == 0) {
         uint32_t v[S / 2];
         if constexpr (S == 4) {
@@ -223,14 +233,29 @@ __device__ __forceinline__ void load_coeffs(const uint16_t *cache, int line, flo
     }
 }
 
-template <int S, typename IdxT, int MT>
+// S planes, MT row tiles (4 batch rows each), a wave owns CT column tiles of 16
+// columns and the workgroup SP sub-groups of K; all CT*SP units of a wave are
+// loaded up front and consumed in order, so the code is straight-line and every
+// wait is for exactly the oldest load.
+// Waves per SIMD the register allocator is asked to leave room for: the queued
+// plane words (and line indices) of all units plus about 70 working registers.
+constexpr int gemv_waves(int S, int MT, int CT, int SP)
+{
+    const int regs = CT * SP * (S + 1) + 56 + 16 * MT + CT * MT + 4 * S;
+    return regs <= 128 ? 4 : (regs <= 168 ? 3 : (regs <= 256 ? 2 : 1));
+}
+
+template <int S, int MT, int CT, int SP, bool TBL>
 __global__ void __launch_bounds__(kThreads)
+__attribute__((amdgpu_waves_per_eu(gemv_waves(S, MT, CT, SP), gemv_waves(S, MT, CT, SP))))
 sbvr_gemv_mfma_kernel(const GemvArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    // smem: A images [SP][MT][64 lanes][32 bytes], then scales [SP][MT*4] floats
+    // smem: A images [SP][MT][64 lanes][32 bytes], scales [SP][MT*4] floats, then
+    // (TBL) a copy of the coefficient table
     unsigned char *img = smem;
-    float *scales = reinterpret_cast<float *>(smem + static_cast<size_t>(a.SP) * MT * 2048);
+    float *scales = reinterpret_cast<float *>(smem + SP * MT * 2048);
+    uint16_t *table = reinterpret_cast<uint16_t *>(smem + SP * MT * 2048 + align16(SP * MT * 16));
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -240,178 +265,237 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     const int N = a.N, K = a.K;
     const int col = lane & 15;   // column inside a tile (B and D operands)
     const int blk = lane >> 4;   // word of the sub-group (B), batch row of the tile (D)
-    const int sg0 = kp * a.SP;   // first sub-group of this workgroup
+    const int sg0 = kp * SP;     // first sub-group of this workgroup
     const int gsub = a.G / kSub; // sub-groups per coefficient group
-    const int U = a.CT * a.SP;   // units (column tile x sub-group) of this wave
-    const int n_wave = (nt * kWavesPerWG + wave) * a.CT * 16;  // first column of this wave
+    const int n_wave = (nt * kWavesPerWG + wave) * CT * 16;  // first column of this wave
 
-    // -- 1. start the weight stream: unit u = (column tile u / SP, sub-group u % SP)
-    Planes<S> q[kPipe];
-    int qline[kPipe];
-    int i_ct = 0, i_sg = 0;      // column tile and sub-group of the next unit to load
-    auto issue = [&](Planes<S> &dst, int &line) {
-        int n = n_wave + i_ct * 16 + col;
-        n = n < N ? n : N - 1;   // clamped lanes compute a value nobody stores
-        const uint32_t word = static_cast<uint32_t>(sg0 + i_sg) * 4 + blk;
-        dst = load_planes<S>(a.bvr + (word * N + n) * S);
-        line = load_idx<IdxT>(a.idx, static_cast<uint32_t>((sg0 + i_sg) / gsub) * N + n);
-        if (++i_sg == a.SP) {
-            i_sg = 0;
-            ++i_ct;
-        }
-    };
+    // -- 1. clear the A images, then issue every global load of the wave, oldest
+    //       first: the activations of its share of the A images, its slice of the
+    //       coefficient table, then the whole weight stream.  Waiting for an early
+    //       load never drains the later ones.
+    for (int i = tid; i < SP * MT * 512; i += kThreads)
+        reinterpret_cast<uint32_t *>(img)[i] = 0u;
+    constexpr int kTasks = SP * MT;          // image tasks per wave, at most (M <= 4*MT)
+    uint32_t xx[kTasks];
 #pragma unroll
-    for (int i = 0; i < kPipe; ++i)
-        if (i < U)
-            issue(q[i], qline[i]);
+    for (int t = 0; t < kTasks; ++t) {
+        const int task = wave + kWavesPerWG * t;     // task = m * SP + sgi
+        const int m = task / SP, sgi = task % SP;
+        const bool valid = m < a.M && !(a.dbg & 4);
+        xx[t] = *reinterpret_cast<const uint32_t *>(
+            a.x + (valid ? static_cast<size_t>(m) * K + static_cast<size_t>(sg0 + sgi) * kSub + 2 * lane : 0));
+    }
+    uint4 treg[kTableRegs];
+    if constexpr (TBL) {
+        // the table is padded to 16 bytes by the host-side contract (a tail of
+        // up to 14 bytes is read, never used): at most kTableRegs uint4 per thread
+        const int vecs = (a.L * S * 2 + 15) / 16;
+#pragma unroll
+        for (int r = 0; r < kTableRegs; ++r) {
+            const int i = tid + r * kThreads;
+            treg[r] = reinterpret_cast<const uint4 *>(a.cache)[i < vecs ? i : 0];
+        }
+    }
+
+    Planes<S> q[SP][CT];
+    int qline[SP][CT];
+#pragma unroll
+    for (int sgi = 0; sgi < SP; ++sgi) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            int n = n_wave + ct * 16 + col;
+            n = n < N ? n : N - 1;   // clamped lanes compute a value nobody stores
+            const uint32_t word = static_cast<uint32_t>(sg0 + sgi) * 4 + blk;
+            if (a.dbg & 16) {
+#pragma unroll
+                for (int j = 0; j < S; ++j)
+                    q[sgi][ct].w[j] = word * 2654435761u + n * 40503u + j;
+            } else
+            q[sgi][ct] = load_planes<S>(a.bvr + (word * N + n) * S);
+            const uint32_t io = static_cast<uint32_t>((sg0 + sgi) / gsub) * N + n;
+            if (a.idx16)
+                qline[sgi][ct] = static_cast<int>(static_cast<const uint16_t *>(a.idx)[io]);
+            else
+                qline[sgi][ct] = static_cast<int>(static_cast<const uint8_t *>(a.idx)[io]);
+        }
+    }
+    if constexpr (TBL) {
+        const int vecs = (a.L * S * 2 + 15) / 16;
+#pragma unroll
+        for (int r = 0; r < kTableRegs; ++r) {
+            const int i = tid + r * kThreads;
+            if (i < vecs)
+                reinterpret_cast<uint4 *>(table)[i] = treg[r];
+        }
+    }
+    __syncthreads();
 
     // -- 2. A images of this workgroup's sub-groups
-    for (int i = tid; i < a.SP * MT * 512; i += kThreads)
-        reinterpret_cast<uint32_t *>(img)[i] = 0u;
-    __syncthreads();
-    for (int task = wave; task < a.SP * a.M; task += kWavesPerWG) {
-        const int sgi = task / a.M, m = task - sgi * a.M;
-        const uint32_t xx = *reinterpret_cast<const uint32_t *>(
-            a.x + static_cast<size_t>(m) * K + static_cast<size_t>(sg0 + sgi) * kSub + 2 * lane);
-        const float x0 = h2f(static_cast<uint16_t>(xx & 0xffffu));
-        const float x1 = h2f(static_cast<uint16_t>(xx >> 16));
-        float amax = fmaxf(fabsf(x0), fabsf(x1));
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1)
-            amax = fmaxf(amax, __shfl_xor(amax, o));
-        // 2^e puts the largest magnitude into [32, 64)
-        const int E = static_cast<int>((__float_as_uint(amax) >> 23) & 255u) - 127;
-        const int e = (amax > 0.f && E < 100) ? 5 - E : 0;
-        const float up = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
-        const int mt = m >> 2, row = (m & 3) * 4;
-        unsigned char *dst = img + static_cast<size_t>(sgi * MT + mt) * 2048;
-        if (lane == 0)   // products come out as 2*x*2^e
-            scales[sgi * (MT * 4) + m] = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
+    for (int t = 0; t < kTasks; ++t) {
+        const int task = wave + kWavesPerWG * t;
+        const int m = task / SP, sgi = task % SP;
+        if (m < a.M && !(a.dbg & 4)) {
+            const float x0 = h2f(static_cast<uint16_t>(xx[t] & 0xffffu));
+            const float x1 = h2f(static_cast<uint16_t>(xx[t] >> 16));
+            float amax = fmaxf(fabsf(x0), fabsf(x1));
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int k = 2 * lane + h;
-            const int t = k & 3;
-            float z = (h ? x1 : x0) * up * (t == 0 ? 4.f : (t == 1 ? 2.f : 1.f));
-            // h1 + h2 + h3/256 == z exactly: each fp8 takes the next 4 significant
-            // bits, the last one of the residual scaled up out of the subnormals
+            for (int o = 32; o > 0; o >>= 1)
+                amax = fmaxf(amax, __shfl_xor(amax, o));
+            // 2^e puts the largest magnitude into [32, 64)
+            const int E = static_cast<int>((__float_as_uint(amax) >> 23) & 255u) - 127;
+            const int e = (amax > 0.f && E < 100) ? 5 - E : 0;
+            const float up = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+            const int mt = m >> 2, row = (m & 3) * 4;
+            unsigned char *dst = img + (sgi * MT + mt) * 2048;
+            if (lane == 0)   // products come out as 2*x*2^e
+                scales[sgi * (MT * 4) + m] = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
 #pragma unroll
-            for (int term = 0; term < 3; ++term) {
-                if (term == 2)
-                    z *= kLastTermScale;
-                const int b = __builtin_amdgcn_cvt_pk_fp8_f32(z, 0.f, 0, false) & 0xff;
-                z -= __builtin_amdgcn_cvt_f32_fp8(b, 0);
-                dst[a_image_byte_offset(k, row + term)] = static_cast<unsigned char>(b);
+            for (int h = 0; h < 2; ++h) {
+                const int k = 2 * lane + h;
+                const int t4 = k & 3;
+                float z = (h ? x1 : x0) * up * (t4 == 0 ? 4.f : (t4 == 1 ? 2.f : 1.f));
+                // h1 + h2 + h3/256 == z exactly: each fp8 takes the next 4 significant
+                // bits, the last one of the residual scaled up out of the subnormals
+#pragma unroll
+                for (int term = 0; term < 3; ++term) {
+                    if (term == 2)
+                        z *= kLastTermScale;
+                    const int b = __builtin_amdgcn_cvt_pk_fp8_f32(z, 0.f, 0, false) & 0xff;
+                    z -= __builtin_amdgcn_cvt_f32_fp8(b, 0);
+                    dst[a_image_byte_offset(k, row + term)] = static_cast<unsigned char>(b);
+                }
             }
         }
     }
     __syncthreads();
 
-    // -- 3. stream the units
-    float y[MT];
+    // -- 3. consume the units: sub-group outer (A operand stays in registers),
+    //       column tile inner
+    float y[CT][MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i)
-        y[i] = 0.f;
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            y[ct][mt] = 0.f;
 
-    auto finish_tile = [&](int ct) {
+#pragma unroll
+    for (int sgi = 0; sgi < SP; ++sgi) {
+        v8i A[MT];
+        float sc[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            A[mt] = *reinterpret_cast<const v8i *>(img + (sgi * MT + mt) * 2048 + lane * 32);
+            sc[mt] = scales[sgi * (MT * 4) + mt * 4 + blk];
+        }
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            const Planes<S> pl = q[sgi][ct];
+            const int line = min(qline[sgi][ct], a.L - 1);
+            if (a.dbg & 8) {
+                uint32_t acc = line;
+#pragma unroll
+                for (int j = 0; j < S; ++j)
+                    acc ^= pl.w[j];
+                y[ct][0] += static_cast<float>(acc);
+                continue;
+            }
+            float c[S];
+            if constexpr (TBL)
+                load_coeffs<S>(static_cast<const uint16_t *>(table), line, c);
+            else
+                load_coeffs<S>(a.cache, line, c);
+            v8i B[S];
+#pragma unroll
+            for (int j = 0; j < S; ++j) {
+                const uint32_t w = pl.w[j];
+                B[j][0] = static_cast<int>(w & 0x11111111u);
+                B[j][1] = static_cast<int>(w & 0x22222222u);
+                B[j][2] = static_cast<int>(w & 0x44444444u);
+                B[j][3] = static_cast<int>((w >> 1) & 0x44444444u);
+                B[j][4] = 0; B[j][5] = 0; B[j][6] = 0; B[j][7] = 0;
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                v4f D[S];
+#pragma unroll
+                for (int j = 0; j < S; ++j) {   // the S products are independent: issued together
+                    const v4f z = {0.f, 0.f, 0.f, 0.f};
+                    D[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[mt], B[j], z, 0, 4, 0, 0, 0, 0);
+                }
+                float acc = 0.f;
+#pragma unroll
+                for (int j = 0; j < S; ++j)
+                    acc = fmaf(c[j], fmaf(D[j][2], 1.f / kLastTermScale, D[j][0] + D[j][1]), acc);
+                y[ct][mt] = fmaf(acc, sc[mt], y[ct][mt]);
+            }
+            // keep the units apart: pin the running sums here, or all MFMAs of the
+            // wave are issued first and their results stay live to the end
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                asm volatile("" : "+v"(y[ct][mt]));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // -- 4. results: direct when K is not split, else through the accumulators
+    if (a.dbg & 2)
+        return;
+    unsigned long long old[CT][MT], adds[CT][MT];
+    if (a.ksplit > 1) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            const int n = n_wave + ct * 16 + col;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m = mt * 4 + blk;
+                old[ct][mt] = 0ull;
+                adds[ct][mt] = 0ull;
+                if (n < N && m < a.M) {
+                    const float v = fminf(fmaxf(y[ct][mt], -kAccClamp), kAccClamp) * static_cast<float>(1 << kAccFracBits);
+                    const long long fx = static_cast<long long>(__builtin_rintf(v)) + kAccBias;
+                    const unsigned long long add = (1ull << 56) + static_cast<unsigned long long>(fx);
+                    old[ct][mt] = __hip_atomic_fetch_add(&a.acc[static_cast<size_t>(m) * N + n], add,
+                                                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    adds[ct][mt] = add;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
         const int n = n_wave + ct * 16 + col;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 4 + blk;
             if (n < N && m < a.M) {
-                if (a.ksplit == 1) {
-                    uint16_t r = f2h(y[mt]);
-                    if (a.bias)
-                        r = hadd(r, a.bias[n]);
-                    a.out[static_cast<size_t>(m) * N + n] = r;
-                } else {
-                    a.partial[(static_cast<size_t>(kp) * a.M + m) * N + n] = y[mt];
+                float total = y[ct][mt];
+                bool mine = true;
+                if (a.ksplit > 1) {
+                    const unsigned long long tot = old[ct][mt] + adds[ct][mt];
+                    mine = static_cast<int>(tot >> 56) == a.ksplit;
+                    if (mine) {
+                        const long long sum = static_cast<long long>(tot & ((1ull << 56) - 1)) -
+                                              static_cast<long long>(a.ksplit) * kAccBias;
+                        total = static_cast<float>(static_cast<double>(sum) * (1.0 / (1 << kAccFracBits)));
+                        __hip_atomic_store(&a.acc[static_cast<size_t>(m) * N + n], 0ull,
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
-            }
-            y[mt] = 0.f;
-        }
-    };
-
-    int p_ct = 0, p_sg = 0;      // column tile and sub-group of the unit being processed
-    auto process = [&](const Planes<S> &pl, int line) {
-        const int ct = p_ct, sgi = p_sg;
-        float c[S];
-        load_coeffs<S>(a.cache, min(line, a.L - 1), c);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const v8i A = *reinterpret_cast<const v8i *>(img + static_cast<size_t>(sgi * MT + mt) * 2048 + lane * 32);
-            const float sc = scales[sgi * (MT * 4) + mt * 4 + blk];
-            float acc = 0.f;
-#pragma unroll
-            for (int j = 0; j < S; ++j) {
-                const uint32_t w = pl.w[j];
-                v8i B;
-                B[0] = static_cast<int>(w & 0x11111111u);
-                B[1] = static_cast<int>(w & 0x22222222u);
-                B[2] = static_cast<int>(w & 0x44444444u);
-                B[3] = static_cast<int>((w >> 1) & 0x44444444u);
-                B[4] = 0; B[5] = 0; B[6] = 0; B[7] = 0;
-                const v4f z = {0.f, 0.f, 0.f, 0.f};
-                const v4f D = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, z, 0, 4, 0, 0, 0, 0);
-                acc = fmaf(c[j], fmaf(D[2], 1.f / kLastTermScale, D[0] + D[1]), acc);
-            }
-            y[mt] = fmaf(acc, sc, y[mt]);
-        }
-        if (++p_sg == a.SP) {
-            p_sg = 0;
-            ++p_ct;
-            finish_tile(ct);
-        }
-    };
-
-    for (int u0 = 0; u0 < U; u0 += kPipe) {
-#pragma unroll
-        for (int i = 0; i < kPipe; ++i) {
-            const int u = u0 + i;
-            if (u < U) {
-                const Planes<S> pl = q[i];
-                const int line = qline[i];
-                if (u + kPipe < U)
-                    issue(q[i], qline[i]);
-                process(pl, line);
-            }
-        }
-    }
-
-    // -- 4. split K: the last workgroup of a column tile adds the partial sums
-    if (a.ksplit > 1) {
-        __shared__ int s_last;
-        __threadfence();
-        __syncthreads();
-        if (tid == 0) {
-            const unsigned prev = atomicAdd(&a.counters[nt], 1u);
-            s_last = (prev == static_cast<unsigned>(a.ksplit - 1));
-        }
-        __syncthreads();
-        if (s_last) {
-            __threadfence();
-            const int cols = kWavesPerWG * a.CT * 16;
-            const int n0 = nt * cols;
-            for (int i = tid; i < cols * a.M; i += kThreads) {
-                const int m = i / cols, n = n0 + (i - m * cols);
-                if (n < N) {
-                    float s = 0.f;
-                    for (int p = 0; p < a.ksplit; ++p)
-                        s += a.partial[(static_cast<size_t>(p) * a.M + m) * N + n];
-                    uint16_t r = f2h(s);
+                if (mine) {
+                    uint16_t r = f2h(total);
                     if (a.bias)
                         r = hadd(r, a.bias[n]);
                     a.out[static_cast<size_t>(m) * N + n] = r;
                 }
             }
-            if (tid == 0)
-                a.counters[nt] = 0u;
         }
     }
 }
 
 // Launch shape for the MFMA kernel.
 struct GemvPlan {
-    int CT, SP, n_tiles, ksplit, MT;
+    int CT, SP, n_tiles, ksplit, MT, table_in_lds;
     size_t lds;
 };
 
@@ -421,77 +505,111 @@ int env_int(const char *name, int dflt)
     return v && *v ? atoi(v) : dflt;
 }
 
-GemvPlan plan_gemv(int M, int N, int K, int cus)
+// (CT, SP) pairs that have a kernel instance; see the dispatch below.
+constexpr int kShapes[][2] = {{1, 1}, {2, 1}, {4, 1}, {8, 1}, {2, 2}, {4, 2}, {8, 2}, {2, 4}, {4, 4}, {1, 8}, {2, 8}};
+constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
+
+bool shape_ok_for(int MT, int CT, int SP)
+{
+    // larger batches keep to the smaller unit counts (register budget)
+    return MT == 1 || CT * SP <= 8;
+}
+
+GemvPlan plan_gemv(int M, int N, int K, int S, int L, int cus)
 {
     const int nsub = K / kSub;
-    const int MT = (M + 3) / 4;
+    const int MT = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
     const int tiles16 = (N + 15) / 16;
     GemvPlan best{};
     double best_cost = 1e30;
-    for (int SP = 1; SP <= nsub && SP <= 8; ++SP) {
-        if (nsub % SP)
+    const int eCT = env_int("SBVR_HIP_CT", 0), eSP = env_int("SBVR_HIP_SP", 0);
+    for (int i = 0; i < kNumShapes; ++i) {
+        const int CT = kShapes[i][0], SP = kShapes[i][1];
+        if (nsub % SP || !shape_ok_for(MT, CT, SP) || nsub / SP > kMaxKsplit)
             continue;
-        for (int CT = 1; CT <= 8; ++CT) {
-            const int U = CT * SP;
-            if (U > 16)
-                continue;
-            const int n_tiles = (tiles16 + kWavesPerWG * CT - 1) / (kWavesPerWG * CT);
-            const int ksplit = nsub / SP;
-            const long wgs = static_cast<long>(n_tiles) * ksplit;
-            // two workgroups per CU run at once; every workgroup pays a fixed
-            // start-up (about 6 units' worth) and its share of the A images
-            const double rounds = static_cast<double>((wgs + 2L * cus - 1) / (2L * cus));
-            const double per_wg = U + 6.0 + 0.5 * SP * M;
-            const double waste = static_cast<double>(n_tiles) * kWavesPerWG * CT / tiles16;
-            const double cost = rounds * per_wg * waste + 0.02 * ksplit;
-            if (cost < best_cost) {
-                best_cost = cost;
-                best = GemvPlan{CT, SP, n_tiles, ksplit, MT, 0};
-            }
+        if (eCT > 0 && eSP > 0 && (CT != eCT || SP != eSP))
+            continue;
+        const int U = CT * SP;
+        const int n_tiles = (tiles16 + kWavesPerWG * CT - 1) / (kWavesPerWG * CT);
+        const int ksplit = nsub / SP;
+        const double wgs = static_cast<double>(n_tiles) * ksplit;
+        // A workgroup puts one wave on each SIMD, so `occ` workgroups fit a CU.
+        // Work that does not fit runs in a second round, which costs the whole
+        // start-up latency again: plans that fit in one round win.  Within a
+        // round every wave pays a fixed start-up (~4 units) and its share of
+        // the A images (~1.5 units per sub-group and batch row).
+        const int occ = gemv_waves(S, MT, CT, SP);
+        const double rounds = static_cast<double>((static_cast<long>(wgs) + static_cast<long>(cus) * occ - 1) /
+                                                  (static_cast<long>(cus) * occ));
+        const double per_wave = U + 4.0 + 1.5 * SP * M / kWavesPerWG;
+        const double waste = static_cast<double>(n_tiles) * kWavesPerWG * CT / tiles16;
+        const double fill = wgs < 1.5 * cus ? 1.5 * cus / wgs : 1.0;   // too few waves to cover latency
+        const double cost = rounds * (per_wave * waste / U * fill + 4.0 / U) + 0.01 * ksplit;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = GemvPlan{CT, SP, n_tiles, ksplit, MT, 0, 0};
         }
     }
-    const int eCT = env_int("SBVR_HIP_CT", 0), eSP = env_int("SBVR_HIP_SP", 0);
-    if (eCT > 0 && eSP > 0 && nsub % eSP == 0) {
-        best.CT = eCT;
-        best.SP = eSP;
-        best.n_tiles = (tiles16 + kWavesPerWG * eCT - 1) / (kWavesPerWG * eCT);
-        best.ksplit = nsub / eSP;
-    }
-    best.MT = MT;
-    best.lds = static_cast<size_t>(best.SP) * MT * 2048 + static_cast<size_t>(best.SP) * MT * 4 * sizeof(float);
+    best.lds = static_cast<size_t>(best.SP) * MT * 2048 + align16(static_cast<size_t>(best.SP) * MT * 16);
+    const size_t table = align16(static_cast<size_t>(L) * S * sizeof(uint16_t));
+    best.table_in_lds = table <= kMaxTableLds && (static_cast<size_t>(L) * S) % 8 == 0;
+    if (best.table_in_lds)
+        best.lds += table;
     return best;
 }
 
 bool mfma_path_ok(int M, int N, int K, int S, int G)
 {
-    // 32-bit element offsets into bvr; one counter per workgroup column tile
-    return M >= 1 && M <= 4 * kMaxMT && K % kSub == 0 && G % kSub == 0 &&
+    // 32-bit element offsets into bvr
+    return M >= 1 && M <= kMaxM && K % kSub == 0 && G % kSub == 0 &&
            (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) &&
-           static_cast<double>(K / 32) * N * S < 2147483648.0 && (N + 63) / 64 <= kMaxTiles;
+           static_cast<double>(K / 32) * N * S < 2147483648.0 && K / kSub <= kMaxKsplit;
 }
 
-template <int S, typename IdxT>
-hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
+template <int S, int MT, int CT, int SP>
+hipError_t launch_gemv_inst(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
     const dim3 grid(static_cast<unsigned>(p.n_tiles) * p.ksplit), block(kThreads);
-    switch (p.MT) {
-    case 1: hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, IdxT, 1>), grid, block, p.lds, st, a); break;
-    case 2: hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, IdxT, 2>), grid, block, p.lds, st, a); break;
-    case 3: hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, IdxT, 3>), grid, block, p.lds, st, a); break;
-    default: hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, IdxT, 4>), grid, block, p.lds, st, a); break;
-    }
+    if (p.table_in_lds)
+        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, true>), grid, block, p.lds, st, a);
+    else
+        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, false>), grid, block, p.lds, st, a);
     return hipGetLastError();
 }
 
-template <typename IdxT>
-hipError_t launch_gemv_s(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t st)
+template <int S, int MT>
+hipError_t launch_gemv_shape(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
+{
+#define SBVR_SHAPE(ct, sp)                  \
+    if (p.CT == ct && p.SP == sp)           \
+        return launch_gemv_inst<S, MT, ct, sp>(a, p, st)
+    SBVR_SHAPE(1, 1); SBVR_SHAPE(2, 1); SBVR_SHAPE(4, 1); SBVR_SHAPE(8, 1);
+    SBVR_SHAPE(2, 2); SBVR_SHAPE(4, 2); SBVR_SHAPE(2, 4); SBVR_SHAPE(1, 8);
+    if constexpr (MT == 1) {
+        SBVR_SHAPE(8, 2); SBVR_SHAPE(4, 4); SBVR_SHAPE(2, 8);
+    }
+#undef SBVR_SHAPE
+    return hipErrorInvalidConfiguration;
+}
+
+template <int S>
+hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
+{
+    switch (p.MT) {
+    case 1: return launch_gemv_shape<S, 1>(a, p, st);
+    case 2: return launch_gemv_shape<S, 2>(a, p, st);
+    default: return launch_gemv_shape<S, 4>(a, p, st);
+    }
+}
+
+hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
     switch (S) {
-    case 2: return launch_gemv_mt<2, IdxT>(a, p, st);
-    case 3: return launch_gemv_mt<3, IdxT>(a, p, st);
-    case 4: return launch_gemv_mt<4, IdxT>(a, p, st);
-    case 6: return launch_gemv_mt<6, IdxT>(a, p, st);
-    default: return launch_gemv_mt<8, IdxT>(a, p, st);
+    case 2: return launch_gemv_mt<2>(a, p, st);
+    case 3: return launch_gemv_mt<3>(a, p, st);
+    case 4: return launch_gemv_mt<4>(a, p, st);
+    case 6: return launch_gemv_mt<6>(a, p, st);
+    default: return launch_gemv_mt<8>(a, p, st);
     }
 }
 
@@ -608,9 +726,7 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G)
 {
     if (!mfma_path_ok(M, N, K, S, G))
         return 0;
-    // the plan depends on the CU count; size for the worst case over plans:
-    // the counter area + ksplit*M*N floats with ksplit <= K/128
-    return kCounterBytes + static_cast<size_t>(K / kSub) * M * N * sizeof(float);
+    return static_cast<size_t>(M) * N * sizeof(unsigned long long);
 }
 
 int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_idx,
@@ -636,7 +752,7 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
     const bool aligned = reinterpret_cast<uintptr_t>(bvr) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(coeff_cache) % 16 == 0;
     if (!(flags & 1) && aligned && mfma_path_ok(M, N, K, S, G)) {
-        const GemvPlan p = plan_gemv(M, N, K, current_cus());
+        const GemvPlan p = plan_gemv(M, N, K, S, L, current_cus());
         GemvArgs a{};
         a.x = static_cast<const uint16_t *>(x);
         a.bvr = bvr;
@@ -645,18 +761,19 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
         a.bias = static_cast<const uint16_t *>(bias);
         a.out = static_cast<uint16_t *>(out);
         a.M = M; a.N = N; a.K = K; a.G = G; a.L = L;
-        a.CT = p.CT; a.SP = p.SP; a.n_tiles = p.n_tiles; a.ksplit = p.ksplit;
+        a.idx16 = idx_bytes == 2;
+        a.n_tiles = p.n_tiles; a.ksplit = p.ksplit; a.table_in_lds = p.table_in_lds; a.dbg = flags;
         if (p.ksplit > 1) {
-            const size_t counters = kCounterBytes;
-            const size_t need = counters + static_cast<size_t>(p.ksplit) * M * N * sizeof(float);
+            const size_t need = static_cast<size_t>(M) * N * sizeof(unsigned long long);
             if (!workspace || workspace_bytes < need)
                 return fail(SBVR_HIP_EWORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-            a.counters = static_cast<unsigned *>(workspace);
-            a.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + counters);
+            if (reinterpret_cast<uintptr_t>(workspace) % 8 != 0)
+                return fail(SBVR_HIP_EINVAL, "workspace must be 8-byte aligned");
+            a.acc = static_cast<unsigned long long *>(workspace);
         }
-        const hipError_t e = (idx_bytes == 1) ? launch_gemv_s<uint8_t>(S, a, p, st) : launch_gemv_s<uint16_t>(S, a, p, st);
+        const hipError_t e = launch_gemv(S, a, p, st);
         if (e != hipSuccess)
-            return fail(SBVR_HIP_ELAUNCH, "gemv launch: %s", hipGetErrorString(e));
+            return fail(SBVR_HIP_ELAUNCH, "gemv launch (CT=%d SP=%d MT=%d): %s", p.CT, p.SP, p.MT, hipGetErrorString(e));
         return SBVR_HIP_OK;
     }
 
