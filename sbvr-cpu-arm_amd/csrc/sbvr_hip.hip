@@ -147,14 +147,25 @@ struct GemvArgs {
     uint16_t *out;
     unsigned long long *acc;   // (M, N) split-K accumulators, all zero between calls
     int M, N, K, G, L;
-    int idx16;            // coeff_idx holds uint16 (else uint8)
     int n_tiles;          // workgroups along N
     int ksplit;           // workgroups along K
-    int table_in_lds;     // coefficient table copied to LDS
-    int dbg;
+#ifdef SBVR_TRACE
+    unsigned long long *trace;   // 8 timestamps per workgroup (development builds only)
+#endif
 };
 
 __host__ __device__ constexpr size_t align16(size_t v) { return (v + 15) & ~static_cast<size_t>(15); }
+
+#ifdef SBVR_TRACE
+#define SBVR_STAMP(i)                                                         \
+    do {                                                                      \
+        if (a.trace && threadIdx.x == 0)                                      \
+            a.trace[blockIdx.x * 8 + (i)] = wall_clock64();                   \
+    } while (0)
+unsigned long long *g_trace = nullptr;
+#else
+#define SBVR_STAMP(i) do { } while (0)
+#endif
 
 // Where element k (0..127) of row `row` (0..15) of a sub-group sits in the A
 // operand of v_mfma_f32_16x16x128_f8f6f4 with fp8 A and fp4 B, given that B
@@ -169,6 +180,9 @@ __device__ __forceinline__ int a_image_byte_offset(int k, int row)
     const int lane = 16 * ((kk >> 4) & 3) + row;
     return lane * 32 + p;
 }
+
+template <bool Wide> struct IdxType { typedef uint8_t type; };
+template <> struct IdxType<true> { typedef uint16_t type; };
 
 template <int S>
 struct Planes {
@@ -238,18 +252,50 @@ __device__ __forceinline__ void load_coeffs(P cache, int line, float (&c)[S])
 // loaded up front and consumed in order, so the code is straight-line and every
 // wait is for exactly the oldest load.
 // Waves per SIMD the register allocator is asked to leave room for: the queued
-// plane words (and line indices) of all units plus about 70 working registers.
+// plane words (and line indices) of all units plus the working registers.
 constexpr int gemv_waves(int S, int MT, int CT, int SP)
 {
-    const int regs = CT * SP * (S + 1) + 56 + 16 * MT + CT * MT + 4 * S;
-    return regs <= 128 ? 4 : (regs <= 168 ? 3 : (regs <= 256 ? 2 : 1));
+    // queued units, double-buffered products, A operands, sums, coefficients, scratch
+    const int regs = CT * SP * (S + 1) + 8 * MT * S + 8 * MT + CT * MT + S + (S < 4 ? 20 : 4);
+    const int w = 512 / regs;
+    return w < 1 ? 1 : (w > 8 ? 8 : w);
 }
 
-template <int S, int MT, int CT, int SP, bool TBL>
+// max over the 64 lanes of a non-negative integer; the result is wave-uniform
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v)
+{
+    v = max(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, true)));   // quad_perm 1,0,3,2
+    v = max(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, true)));   // quad_perm 2,3,0,1
+    v = max(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x141, 0xF, 0xF, true)));  // row_half_mirror
+    v = max(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x140, 0xF, 0xF, true)));  // row_mirror
+    const uint32_t r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
+    const uint32_t r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
+    return max(max(r0, r1), max(r2, r3));
+}
+
+// float -> the split-K accumulator's fixed point (2^-kAccFracBits), |v| <= kAccClamp.
+// hi = rint(y * 2^(F-24)) and lo = y * 2^F - hi * 2^24 are exact in fp32.
+__device__ __forceinline__ long long to_fixed(float y)
+{
+    y = fminf(fmaxf(y, -kAccClamp), kAccClamp);
+    const float hi = __builtin_rintf(y * static_cast<float>(1 << (kAccFracBits - 24)));
+    const float lo = fmaf(hi, -16777216.f, y * static_cast<float>(1 << kAccFracBits));
+    return (static_cast<long long>(static_cast<int>(hi)) << 24) + static_cast<long long>(static_cast<int>(lo));
+}
+
+// MODE 0: table in LDS, uint8 indices; 1: table in LDS, uint16 indices;
+//      2: table read from global memory (large tables), uint16 indices.
+// S planes, MT row tiles (4 batch rows each); a wave owns CT column tiles of 16
+// columns and the workgroup SP sub-groups of K.  All CT*SP units of a wave are
+// loaded up front and consumed in order: the code is straight-line, every wait
+// is for exactly the oldest load, and addresses are one base plus immediates.
+template <int S, int MT, int CT, int SP, int MODE>
 __global__ void __launch_bounds__(kThreads)
 __attribute__((amdgpu_waves_per_eu(gemv_waves(S, MT, CT, SP), gemv_waves(S, MT, CT, SP))))
 sbvr_gemv_mfma_kernel(const GemvArgs a)
 {
+    constexpr bool TBL = MODE != 2;
+    typedef typename IdxType<MODE != 0>::type IdxT;
     extern __shared__ __align__(16) unsigned char smem[];
     // smem: A images [SP][MT][64 lanes][32 bytes], scales [SP][MT*4] floats, then
     // (TBL) a copy of the coefficient table
@@ -267,8 +313,13 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     const int blk = lane >> 4;   // word of the sub-group (B), batch row of the tile (D)
     const int sg0 = kp * SP;     // first sub-group of this workgroup
     const int gsub = a.G / kSub; // sub-groups per coefficient group
-    const int n_wave = (nt * kWavesPerWG + wave) * CT * 16;  // first column of this wave
+    // The wave owns columns [n_own, n_own + 16*CT).  It computes a full window
+    // of 16*CT columns; a window that would stick out of N is moved left, and
+    // the columns it then shares with its neighbour are left to the neighbour.
+    const int n_own = (nt * kWavesPerWG + wave) * CT * 16;
+    const int n_base = min(n_own, N - CT * 16);
 
+    SBVR_STAMP(0);
     // -- 1. clear the A images, then issue every global load of the wave, oldest
     //       first: the activations of its share of the A images, its slice of the
     //       coefficient table, then the whole weight stream.  Waiting for an early
@@ -281,97 +332,92 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     for (int t = 0; t < kTasks; ++t) {
         const int task = wave + kWavesPerWG * t;     // task = m * SP + sgi
         const int m = task / SP, sgi = task % SP;
-        const bool valid = m < a.M && !(a.dbg & 4);
         xx[t] = *reinterpret_cast<const uint32_t *>(
-            a.x + (valid ? static_cast<size_t>(m) * K + static_cast<size_t>(sg0 + sgi) * kSub + 2 * lane : 0));
+            a.x + (m < a.M ? static_cast<size_t>(m) * K + static_cast<size_t>(sg0 + sgi) * kSub + 2 * lane : 0));
     }
     uint4 treg[kTableRegs];
+    const int tvecs = a.L * S / 8;           // the table is a whole number of 16-byte vectors here
     if constexpr (TBL) {
-        // the table is padded to 16 bytes by the host-side contract (a tail of
-        // up to 14 bytes is read, never used): at most kTableRegs uint4 per thread
-        const int vecs = (a.L * S * 2 + 15) / 16;
 #pragma unroll
         for (int r = 0; r < kTableRegs; ++r) {
             const int i = tid + r * kThreads;
-            treg[r] = reinterpret_cast<const uint4 *>(a.cache)[i < vecs ? i : 0];
+            treg[r] = reinterpret_cast<const uint4 *>(a.cache)[i < tvecs ? i : 0];
         }
     }
 
     Planes<S> q[SP][CT];
     int qline[SP][CT];
+    {
+        const uint32_t lane_w = (static_cast<uint32_t>(blk) * N + n_base + col) * S;   // words
+        const uint32_t lane_i = static_cast<uint32_t>(n_base + col);
 #pragma unroll
-    for (int sgi = 0; sgi < SP; ++sgi) {
+        for (int sgi = 0; sgi < SP; ++sgi) {
+            const uint32_t *wrow = a.bvr + static_cast<size_t>(sg0 + sgi) * 4 * N * S;     // wave-uniform
+            const IdxT *irow = static_cast<const IdxT *>(a.idx) + static_cast<size_t>((sg0 + sgi) / gsub) * N;
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            int n = n_wave + ct * 16 + col;
-            n = n < N ? n : N - 1;   // clamped lanes compute a value nobody stores
-            const uint32_t word = static_cast<uint32_t>(sg0 + sgi) * 4 + blk;
-            if (a.dbg & 16) {
-#pragma unroll
-                for (int j = 0; j < S; ++j)
-                    q[sgi][ct].w[j] = word * 2654435761u + n * 40503u + j;
-            } else
-            q[sgi][ct] = load_planes<S>(a.bvr + (word * N + n) * S);
-            const uint32_t io = static_cast<uint32_t>((sg0 + sgi) / gsub) * N + n;
-            if (a.idx16)
-                qline[sgi][ct] = static_cast<int>(static_cast<const uint16_t *>(a.idx)[io]);
-            else
-                qline[sgi][ct] = static_cast<int>(static_cast<const uint8_t *>(a.idx)[io]);
+            for (int ct = 0; ct < CT; ++ct) {
+                q[sgi][ct] = load_planes<S>(wrow + lane_w + ct * 16 * S);
+                qline[sgi][ct] = static_cast<int>(irow[lane_i + ct * 16]);
+            }
         }
     }
     if constexpr (TBL) {
-        const int vecs = (a.L * S * 2 + 15) / 16;
 #pragma unroll
         for (int r = 0; r < kTableRegs; ++r) {
             const int i = tid + r * kThreads;
-            if (i < vecs)
+            if (i < tvecs)
                 reinterpret_cast<uint4 *>(table)[i] = treg[r];
         }
     }
+    SBVR_STAMP(1);
     __syncthreads();
+    SBVR_STAMP(2);
 
-    // -- 2. A images of this workgroup's sub-groups
+    // -- 2. A images of this workgroup's sub-groups: lane l turns elements 2l and
+    //       2l+1 of a (batch row, sub-group) into 3 fp8 terms each
+    {
+        // position of the lane's two elements in an image, and their B-nibble factors
+        const int off0 = a_image_byte_offset(2 * lane, 0), off1 = a_image_byte_offset(2 * lane + 1, 0);
+        const float fac0 = (lane & 1) ? 1.f : 4.f, fac1 = (lane & 1) ? 1.f : 2.f;
 #pragma unroll
-    for (int t = 0; t < kTasks; ++t) {
-        const int task = wave + kWavesPerWG * t;
-        const int m = task / SP, sgi = task % SP;
-        if (m < a.M && !(a.dbg & 4)) {
-            const float x0 = h2f(static_cast<uint16_t>(xx[t] & 0xffffu));
-            const float x1 = h2f(static_cast<uint16_t>(xx[t] >> 16));
-            float amax = fmaxf(fabsf(x0), fabsf(x1));
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1)
-                amax = fmaxf(amax, __shfl_xor(amax, o));
-            // 2^e puts the largest magnitude into [32, 64)
-            const int E = static_cast<int>((__float_as_uint(amax) >> 23) & 255u) - 127;
-            const int e = (amax > 0.f && E < 100) ? 5 - E : 0;
-            const float up = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
-            const int mt = m >> 2, row = (m & 3) * 4;
-            unsigned char *dst = img + (sgi * MT + mt) * 2048;
-            if (lane == 0)   // products come out as 2*x*2^e
-                scales[sgi * (MT * 4) + m] = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int k = 2 * lane + h;
-                const int t4 = k & 3;
-                float z = (h ? x1 : x0) * up * (t4 == 0 ? 4.f : (t4 == 1 ? 2.f : 1.f));
+        for (int t = 0; t < kTasks; ++t) {
+            const int task = wave + kWavesPerWG * t;
+            const int m = task / SP, sgi = task % SP;
+            if (m < a.M) {
+                // 2^e puts the largest magnitude of the sub-group into [32, 64)
+                // (fp16 bits order like magnitudes; subnormals count as 2^-15)
+                const uint32_t amax = wave_umax(max(xx[t] & 0x7fffu, (xx[t] >> 16) & 0x7fffu));
+                const int eh = min(max(static_cast<int>(amax >> 10), 1), 30);
+                const int e = 20 - eh;
+                const float up = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+                unsigned char *dst = img + (sgi * MT + (m >> 2)) * 2048 + (m & 3) * 4 * 32;
+                if (lane == 0)   // products come out as 2 * x * 2^e
+                    scales[sgi * (MT * 4) + m] = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
+                float z0 = h2f(static_cast<uint16_t>(xx[t] & 0xffffu)) * (up * fac0);
+                float z1 = h2f(static_cast<uint16_t>(xx[t] >> 16)) * (up * fac1);
                 // h1 + h2 + h3/256 == z exactly: each fp8 takes the next 4 significant
                 // bits, the last one of the residual scaled up out of the subnormals
 #pragma unroll
                 for (int term = 0; term < 3; ++term) {
-                    if (term == 2)
-                        z *= kLastTermScale;
-                    const int b = __builtin_amdgcn_cvt_pk_fp8_f32(z, 0.f, 0, false) & 0xff;
-                    z -= __builtin_amdgcn_cvt_f32_fp8(b, 0);
-                    dst[a_image_byte_offset(k, row + term)] = static_cast<unsigned char>(b);
+                    if (term == 2) {
+                        z0 *= kLastTermScale;
+                        z1 *= kLastTermScale;
+                    }
+                    const int b = __builtin_amdgcn_cvt_pk_fp8_f32(z0, z1, 0, false);
+                    z0 -= __builtin_amdgcn_cvt_f32_fp8(b, 0);
+                    z1 -= __builtin_amdgcn_cvt_f32_fp8(b, 1);
+                    dst[off0 + term * 32] = static_cast<unsigned char>(b & 0xff);
+                    dst[off1 + term * 32] = static_cast<unsigned char>((b >> 8) & 0xff);
                 }
             }
         }
     }
     __syncthreads();
+    SBVR_STAMP(3);
 
     // -- 3. consume the units: sub-group outer (A operand stays in registers),
-    //       column tile inner
+    //       column tile inner.  The MFMAs of a unit are issued before the
+    //       results of the previous unit are folded in, so their latency is covered.
     float y[CT][MT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
@@ -379,123 +425,132 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
         for (int mt = 0; mt < MT; ++mt)
             y[ct][mt] = 0.f;
 
+    v8i A[MT];
+    float sc[MT];
+    v4f D[2][MT][S];
+    float cprev[S];
+    float scprev[MT];
+    auto products = [&](int sgi, int ct, v4f (&Dn)[MT][S]) {
+        const Planes<S> &pl = q[sgi][ct];
 #pragma unroll
-    for (int sgi = 0; sgi < SP; ++sgi) {
-        v8i A[MT];
-        float sc[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            A[mt] = *reinterpret_cast<const v8i *>(img + (sgi * MT + mt) * 2048 + lane * 32);
-            sc[mt] = scales[sgi * (MT * 4) + mt * 4 + blk];
-        }
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            const Planes<S> pl = q[sgi][ct];
-            const int line = min(qline[sgi][ct], a.L - 1);
-            if (a.dbg & 8) {
-                uint32_t acc = line;
-#pragma unroll
-                for (int j = 0; j < S; ++j)
-                    acc ^= pl.w[j];
-                y[ct][0] += static_cast<float>(acc);
-                continue;
-            }
-            float c[S];
-            if constexpr (TBL)
-                load_coeffs<S>(static_cast<const uint16_t *>(table), line, c);
-            else
-                load_coeffs<S>(a.cache, line, c);
-            v8i B[S];
-#pragma unroll
-            for (int j = 0; j < S; ++j) {
-                const uint32_t w = pl.w[j];
-                B[j][0] = static_cast<int>(w & 0x11111111u);
-                B[j][1] = static_cast<int>(w & 0x22222222u);
-                B[j][2] = static_cast<int>(w & 0x44444444u);
-                B[j][3] = static_cast<int>((w >> 1) & 0x44444444u);
-                B[j][4] = 0; B[j][5] = 0; B[j][6] = 0; B[j][7] = 0;
-            }
+        for (int j = 0; j < S; ++j) {
+            const uint32_t w = pl.w[j];
+            v8i B;
+            B[0] = static_cast<int>(w & 0x11111111u);
+            B[1] = static_cast<int>(w & 0x22222222u);
+            B[2] = static_cast<int>(w & 0x44444444u);
+            B[3] = static_cast<int>((w >> 1) & 0x44444444u);
+            B[4] = 0; B[5] = 0; B[6] = 0; B[7] = 0;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                v4f D[S];
-#pragma unroll
-                for (int j = 0; j < S; ++j) {   // the S products are independent: issued together
-                    const v4f z = {0.f, 0.f, 0.f, 0.f};
-                    D[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[mt], B[j], z, 0, 4, 0, 0, 0, 0);
-                }
-                float acc = 0.f;
-#pragma unroll
-                for (int j = 0; j < S; ++j)
-                    acc = fmaf(c[j], fmaf(D[j][2], 1.f / kLastTermScale, D[j][0] + D[j][1]), acc);
-                y[ct][mt] = fmaf(acc, sc[mt], y[ct][mt]);
+                const v4f z = {0.f, 0.f, 0.f, 0.f};
+                Dn[mt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[mt], B, z, 0, 4, 0, 0, 0, 0);
             }
-            // keep the units apart: pin the running sums here, or all MFMAs of the
-            // wave are issued first and their results stay live to the end
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-                asm volatile("" : "+v"(y[ct][mt]));
-            __builtin_amdgcn_sched_barrier(0);
         }
+    };
+    auto coeffs_of = [&](int sgi, int ct, float (&c)[S]) {
+        const int line = min(qline[sgi][ct], a.L - 1);
+        if constexpr (TBL)
+            load_coeffs<S>(static_cast<const uint16_t *>(table), line, c);
+        else
+            load_coeffs<S>(a.cache, line, c);
+    };
+    auto fold = [&](int ct, const v4f (&Dp)[MT][S]) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < S; ++j)
+                acc = fmaf(cprev[j], fmaf(Dp[mt][j][2], 1.f / kLastTermScale, Dp[mt][j][0] + Dp[mt][j][1]), acc);
+            y[ct][mt] = fmaf(acc, scprev[mt], y[ct][mt]);
+            asm volatile("" : "+v"(y[ct][mt]));   // keeps the units in program order
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < SP * CT; ++u) {
+        const int sgi = u / CT, ct = u % CT;
+        if (ct == 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                A[mt] = *reinterpret_cast<const v8i *>(img + (sgi * MT + mt) * 2048 + lane * 32);
+                sc[mt] = scales[sgi * (MT * 4) + mt * 4 + blk];
+            }
+        }
+        float c[S];
+        coeffs_of(sgi, ct, c);
+        products(sgi, ct, D[u & 1]);
+        if (u > 0)
+            fold((u - 1) % CT, D[(u - 1) & 1]);
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+            cprev[j] = c[j];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            scprev[mt] = sc[mt];
+        __builtin_amdgcn_sched_barrier(0);
     }
+    fold((SP * CT - 1) % CT, D[(SP * CT - 1) & 1]);
 
+    SBVR_STAMP(4);
     // -- 4. results: direct when K is not split, else through the accumulators
-    if (a.dbg & 2)
-        return;
-    unsigned long long old[CT][MT], adds[CT][MT];
-    if (a.ksplit > 1) {
+    if (a.ksplit == 1) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            const int n = n_wave + ct * 16 + col;
+            const int n = n_base + ct * 16 + col;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 const int m = mt * 4 + blk;
-                old[ct][mt] = 0ull;
-                adds[ct][mt] = 0ull;
-                if (n < N && m < a.M) {
-                    const float v = fminf(fmaxf(y[ct][mt], -kAccClamp), kAccClamp) * static_cast<float>(1 << kAccFracBits);
-                    const long long fx = static_cast<long long>(__builtin_rintf(v)) + kAccBias;
-                    const unsigned long long add = (1ull << 56) + static_cast<unsigned long long>(fx);
-                    old[ct][mt] = __hip_atomic_fetch_add(&a.acc[static_cast<size_t>(m) * N + n], add,
-                                                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    adds[ct][mt] = add;
-                }
-            }
-        }
-    }
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        const int n = n_wave + ct * 16 + col;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int m = mt * 4 + blk;
-            if (n < N && m < a.M) {
-                float total = y[ct][mt];
-                bool mine = true;
-                if (a.ksplit > 1) {
-                    const unsigned long long tot = old[ct][mt] + adds[ct][mt];
-                    mine = static_cast<int>(tot >> 56) == a.ksplit;
-                    if (mine) {
-                        const long long sum = static_cast<long long>(tot & ((1ull << 56) - 1)) -
-                                              static_cast<long long>(a.ksplit) * kAccBias;
-                        total = static_cast<float>(static_cast<double>(sum) * (1.0 / (1 << kAccFracBits)));
-                        __hip_atomic_store(&a.acc[static_cast<size_t>(m) * N + n], 0ull,
-                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
-                }
-                if (mine) {
-                    uint16_t r = f2h(total);
+                if (n >= n_own && m < a.M) {
+                    uint16_t r = f2h(y[ct][mt]);
                     if (a.bias)
                         r = hadd(r, a.bias[n]);
                     a.out[static_cast<size_t>(m) * N + n] = r;
                 }
             }
         }
+        return;
     }
+    unsigned long long old[CT][MT], adds[CT][MT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int n = n_base + ct * 16 + col;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 4 + blk;
+            old[ct][mt] = 0ull;
+            adds[ct][mt] = (1ull << 56) + static_cast<unsigned long long>(to_fixed(y[ct][mt]) + kAccBias);
+            if (n >= n_own && m < a.M)
+                old[ct][mt] = __hip_atomic_fetch_add(&a.acc[static_cast<size_t>(m) * N + n], adds[ct][mt],
+                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    SBVR_STAMP(5);
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int n = n_base + ct * 16 + col;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 4 + blk;
+            const unsigned long long tot = old[ct][mt] + adds[ct][mt];
+            if (n >= n_own && m < a.M && static_cast<int>(tot >> 56) == a.ksplit) {
+                const long long sum = static_cast<long long>(tot & ((1ull << 56) - 1)) -
+                                      static_cast<long long>(a.ksplit) * kAccBias;
+                const float total = static_cast<float>(static_cast<double>(sum) * (1.0 / (1 << kAccFracBits)));
+                __hip_atomic_store(&a.acc[static_cast<size_t>(m) * N + n], 0ull,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                uint16_t r = f2h(total);
+                if (a.bias)
+                    r = hadd(r, a.bias[n]);
+                a.out[static_cast<size_t>(m) * N + n] = r;
+            }
+        }
+    }
+    SBVR_STAMP(6);
 }
 
 // Launch shape for the MFMA kernel.
 struct GemvPlan {
-    int CT, SP, n_tiles, ksplit, MT, table_in_lds;
+    int CT, SP, n_tiles, ksplit, MT, mode;
     size_t lds;
 };
 
@@ -515,7 +570,7 @@ bool shape_ok_for(int MT, int CT, int SP)
     return MT == 1 || CT * SP <= 8;
 }
 
-GemvPlan plan_gemv(int M, int N, int K, int S, int L, int cus)
+GemvPlan plan_gemv(int M, int N, int K, int S, int L, int idx_bytes, int cus)
 {
     const int nsub = K / kSub;
     const int MT = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
@@ -525,7 +580,7 @@ GemvPlan plan_gemv(int M, int N, int K, int S, int L, int cus)
     const int eCT = env_int("SBVR_HIP_CT", 0), eSP = env_int("SBVR_HIP_SP", 0);
     for (int i = 0; i < kNumShapes; ++i) {
         const int CT = kShapes[i][0], SP = kShapes[i][1];
-        if (nsub % SP || !shape_ok_for(MT, CT, SP) || nsub / SP > kMaxKsplit)
+        if (nsub % SP || !shape_ok_for(MT, CT, SP) || nsub / SP > kMaxKsplit || CT * 16 > N)
             continue;
         if (eCT > 0 && eSP > 0 && (CT != eCT || SP != eSP))
             continue;
@@ -551,17 +606,21 @@ GemvPlan plan_gemv(int M, int N, int K, int S, int L, int cus)
         }
     }
     best.lds = static_cast<size_t>(best.SP) * MT * 2048 + align16(static_cast<size_t>(best.SP) * MT * 16);
-    const size_t table = align16(static_cast<size_t>(L) * S * sizeof(uint16_t));
-    best.table_in_lds = table <= kMaxTableLds && (static_cast<size_t>(L) * S) % 8 == 0;
-    if (best.table_in_lds)
+    const size_t table = static_cast<size_t>(L) * S * sizeof(uint16_t);
+    const bool in_lds = table <= kMaxTableLds && table % 16 == 0;
+    if (in_lds) {
         best.lds += table;
+        best.mode = idx_bytes == 2 ? 1 : 0;
+    } else {
+        best.mode = idx_bytes == 2 ? 2 : -1;   // no kernel for a big table behind uint8 indices (cannot happen: L <= 256)
+    }
     return best;
 }
 
 bool mfma_path_ok(int M, int N, int K, int S, int G)
 {
     // 32-bit element offsets into bvr
-    return M >= 1 && M <= kMaxM && K % kSub == 0 && G % kSub == 0 &&
+    return M >= 1 && M <= kMaxM && N >= 16 && K % kSub == 0 && G % kSub == 0 &&
            (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) &&
            static_cast<double>(K / 32) * N * S < 2147483648.0 && K / kSub <= kMaxKsplit;
 }
@@ -570,10 +629,12 @@ template <int S, int MT, int CT, int SP>
 hipError_t launch_gemv_inst(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
     const dim3 grid(static_cast<unsigned>(p.n_tiles) * p.ksplit), block(kThreads);
-    if (p.table_in_lds)
-        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, true>), grid, block, p.lds, st, a);
+    if (p.mode == 0)
+        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, 0>), grid, block, p.lds, st, a);
+    else if (p.mode == 1)
+        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, 1>), grid, block, p.lds, st, a);
     else
-        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, false>), grid, block, p.lds, st, a);
+        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, 2>), grid, block, p.lds, st, a);
     return hipGetLastError();
 }
 
@@ -698,6 +759,10 @@ sbvr_mm_T_kernel(const uint32_t *__restrict__ l_bvr, const void *__restrict__ l_
 
 extern "C" {
 
+#ifdef SBVR_TRACE
+void sbvr_hip_debug_set_trace(unsigned long long *p) { g_trace = p; }
+#endif
+
 int sbvr_hip_version(void) { return 100; }
 
 const char *sbvr_hip_last_error(void) { return g_err; }
@@ -752,7 +817,8 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
     const bool aligned = reinterpret_cast<uintptr_t>(bvr) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(coeff_cache) % 16 == 0;
     if (!(flags & 1) && aligned && mfma_path_ok(M, N, K, S, G)) {
-        const GemvPlan p = plan_gemv(M, N, K, S, L, current_cus());
+        const GemvPlan p = plan_gemv(M, N, K, S, L, idx_bytes, current_cus());
+        if (p.CT > 0 && p.mode >= 0) {
         GemvArgs a{};
         a.x = static_cast<const uint16_t *>(x);
         a.bvr = bvr;
@@ -761,8 +827,10 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
         a.bias = static_cast<const uint16_t *>(bias);
         a.out = static_cast<uint16_t *>(out);
         a.M = M; a.N = N; a.K = K; a.G = G; a.L = L;
-        a.idx16 = idx_bytes == 2;
-        a.n_tiles = p.n_tiles; a.ksplit = p.ksplit; a.table_in_lds = p.table_in_lds; a.dbg = flags;
+        a.n_tiles = p.n_tiles; a.ksplit = p.ksplit;
+#ifdef SBVR_TRACE
+        a.trace = g_trace;
+#endif
         if (p.ksplit > 1) {
             const size_t need = static_cast<size_t>(M) * N * sizeof(unsigned long long);
             if (!workspace || workspace_bytes < need)
@@ -775,6 +843,7 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "gemv launch (CT=%d SP=%d MT=%d): %s", p.CT, p.SP, p.MT, hipGetErrorString(e));
         return SBVR_HIP_OK;
+        }
     }
 
     const size_t total = static_cast<size_t>(M) * N;

@@ -22,6 +22,10 @@ class SbvrHipError(RuntimeError):
 
 
 def library_path():
+    """The in-tree build, unless SBVR_HIP_LIBRARY names another copy."""
+    override = os.environ.get("SBVR_HIP_LIBRARY")
+    if override:
+        return override
     here = os.path.dirname(os.path.abspath(__file__))
     return os.path.join(os.path.dirname(here), "csrc", _LIB_NAME)
 
