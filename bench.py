@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of the SBVR compressed-domain GEMV on one MI355X.
+
+Workload (BASELINE.json configs[1], the shape the metric is quoted on): the
+Llama-3-8B gate projection 4096 -> 14336 at batch 1, 4 bit planes, group 128,
+uint32-packed planes, fp16 coefficient table of 256 lines (uint8 indices),
+fp16 N(0,1) activations, synthetic seeded encodings.  A step is one GEMV over
+one weight copy; consecutive steps walk through COPIES distinct weight copies
+(about 480 MB) so that every step streams its planes from HBM and not from the
+256 MB Infinity Cache.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+prints one JSON line: whole-job throughput in GB/s of algorithmic bytes, the
+roofline of the kernel (HIP events on the launch stream) and the CPU baseline
+(the x86 port of the reference's timed CPU kernel, on the host's own cores).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "sbvr-cpu-arm_amd"))
+sys.path.insert(0, ROOT)
+
+N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH = 14336, 4096, 4, 128, 256, 1
+COPIES = 16
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(n, k, s, g, lines, m):
+    """Bytes one GEMV has to move: planes + indices + table + activations + outputs."""
+    idx_bytes = 1 if lines <= 256 else 2
+    return n * k * s // 8 + (k // g) * n * idx_bytes + 2 * lines * s + 2 * m * k + 2 * m * n
+
+
+def gpu_leg(steps, warmup):
+    import torch
+    import sbvr
+    from sbvr import synth, hip
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
+    dev = torch.device("cuda:0")
+    sbvr._sbvr_hip_init(dev)
+    weights = []
+    for c in range(COPIES):
+        bvr, idx, cache = synth.random_encoding(N_OUT, K_IN, NUM_SUMS, GROUP, LINES, seed=c)
+        weights.append((bvr.to(dev), idx.to(dev), cache.to(dev)))
+    x = torch.randn((BATCH, K_IN), generator=torch.Generator().manual_seed(1234)).to(torch.float16).to(dev)
+    out = torch.empty((BATCH, N_OUT), dtype=torch.float16, device=dev)
+
+    def step(i):
+        bvr, idx, cache = weights[i % COPIES]
+        hip._sbvr_linear_f16(x, bvr, idx, cache, None, GROUP, out=out)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    # The K timed steps are recorded once into a HIP graph and replayed, so that
+    # the launch path is the driver's and not the Python interpreter's.
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    launcher = "hipGraph"
+    try:
+        with torch.cuda.stream(stream):
+            step(0)                      # workspace for this stream exists before capture
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(steps):
+                    step(warmup + i)
+            graph.replay()               # first replay uploads the graph
+            torch.cuda.synchronize()
+    except Exception as exc:             # capture is an optimisation, not a requirement
+        print(f"bench.py: graph capture failed ({exc}); timing eager launches", file=sys.stderr)
+        graph = None
+        launcher = "eager"
+
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(stream):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                step(warmup + i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    wall_ms = (t1 - t0) * 1e3 / steps
+    event_ms = e0.elapsed_time(e1) / steps
+    return wall_ms, event_ms, launcher, torch.cuda.get_device_name(0)
+
+
+def cpu_leg(budget_s=12.0):
+    """The reference's CPU algorithm (both operands encoded, popcount of AND,
+    fp16 coefficient products) ported to x86, timed on this host for about
+    `budget_s` seconds at the same shape."""
+    import numpy as np
+    from oracle import sbvr_oracle as O
+
+    rng = np.random.default_rng(7)
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    threads = O.PORT.init_pool(threads)
+
+    def planes(rows, s):
+        return rng.integers(0, 256, size=(s, rows * K_IN // 8), dtype=np.uint8)
+
+    s_l = 4
+    l_bvr = O.np_planes_to_default(planes(1, s_l), 1)
+    l_idx = rng.integers(0, 16, size=(K_IN // GROUP, 1)).astype(np.uint8)
+    l_cache = (rng.standard_normal((16, s_l)) * 0.3).astype(np.float16)
+    r_bvr = O.np_planes_to_v1(planes(N_OUT, NUM_SUMS), N_OUT)
+    r_idx = rng.integers(0, LINES, size=(K_IN // GROUP, N_OUT)).astype(np.uint8)
+    r_cache = (rng.standard_normal((LINES, NUM_SUMS)) * 0.02).astype(np.float16)
+    args = (l_bvr, l_idx, l_cache, r_bvr, r_idx, r_cache, GROUP)
+    probe = O.PORT.time_mm_T_v1(*args, warmup=2, iters=3)
+    iters = max(10, int(budget_s / max(probe, 1e-6)))
+    per_call = O.PORT.time_mm_T_v1(*args, warmup=10, iters=iters)
+    O.PORT.finalize_pool()
+    nbytes = algorithmic_bytes(N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH)
+    return {
+        "value": round(nbytes / per_call / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "us_per_gemv": round(per_call * 1e6, 1),
+        "isa": O.PORT.isa(),
+        "sample": f"{iters} timed calls (10 warm-ups) of the full 4096->14336 GEMV, both operands SBVR-encoded "
+                  f"(S_l=4, S_r=4, group 128), reference CPU algorithm ported to x86, N split over {threads} pinned threads",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: the path is single-GPU in this build (run with --gpus 1)")
+
+    wall_ms, event_ms, launcher, device = gpu_leg(a.steps, a.warmup)
+    nbytes = algorithmic_bytes(N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH)
+    value = nbytes / (wall_ms * 1e-3) / 1e9
+    achieved = nbytes / (event_ms * 1e-3) / 1e9
+    line = {
+        "metric": "SBVR GEMV achieved HBM GB/s (%peak) at 4096x14336; 8B decode tokens/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(wall_ms, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "Llama-3-8B gate linear 4096->14336, batch 1, SBVR 4 bit planes, group 128, "
+                        "256 coefficient lines (uint8 idx), fp16 activations",
+            "weight_copies_rotated": COPIES,
+            "bytes_per_step": nbytes,
+            "launcher": launcher,
+            "device": device,
+        },
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "sbvr_gemv_mfma_kernel",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "us_per_launch": round(event_ms * 1e3, 3),
+            "traffic": None,
+        },
+    }
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_leg()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -281,3 +281,71 @@ class _C:
 
 
 C = _C()
+
+
+# ------------------------------------------------------------------ timed CPU port
+
+class _Port:
+    """ctypes view of libsbvr_cpu_port.so: the x86 port of the reference's timed
+    NEON kernel (sbvr_kernel.cpp:251-399, 471-539) with its pinned thread pool.
+    Used as the CPU baseline that bench.py reports beside the GPU figure."""
+
+    def __init__(self):
+        self._lib = None
+
+    @property
+    def lib(self):
+        if self._lib is None:
+            path = os.path.join(_HERE, "libsbvr_cpu_port.so")
+            if not os.path.exists(path):
+                build(targets=("libsbvr_cpu_port.so",))
+            lib = ctypes.CDLL(path)
+            lib.sbvr_port_isa.restype = ctypes.c_char_p
+            lib.sbvr_port_time_mm_T_v1.restype = ctypes.c_double
+            self._lib = lib
+        return self._lib
+
+    def init_pool(self, threads=-1):
+        """-1: one worker per hardware thread, as the reference's import does."""
+        return self.lib.sbvr_port_init_pool(int(threads))
+
+    def finalize_pool(self):
+        self.lib.sbvr_port_finalize_pool()
+
+    def num_threads(self):
+        return self.lib.sbvr_port_num_threads()
+
+    def isa(self):
+        return self.lib.sbvr_port_isa().decode()
+
+    def _args(self, l_bvr, l_idx, l_cache, r_bvr, r_idx, r_cache, G, bias):
+        c = _C._c
+        l_bvr, l_idx, r_bvr, r_idx = c(l_bvr, np.uint8), c(l_idx), c(r_bvr, np.uint8), c(r_idx)
+        l_cache, r_cache = c(l_cache, np.float16), c(r_cache, np.float16)
+        Kb, one, Sl = l_bvr.shape
+        assert one == 1 and r_bvr.ndim == 4 and r_bvr.shape[3] == 16
+        N, Sr = r_bvr.shape[0] * 16, r_bvr.shape[2]
+        b = c(bias, np.float16) if bias is not None and bias.size == N else None
+        out = np.empty((1, N), dtype=np.float16)
+        keep = (l_bvr, l_idx, l_cache, r_bvr, r_idx, r_cache, b, out)
+        args = [_ptr(l_bvr), _ptr(l_idx), l_idx.dtype.itemsize, _ptr(l_cache), _ptr(r_bvr), _ptr(r_idx),
+                r_idx.dtype.itemsize, _ptr(r_cache), _ptr(b), _ptr(out), N, Kb * 8, Sl, Sr, G]
+        return args, out, keep
+
+    def mm_T_v1(self, l_bvr, l_idx, l_cache, r_bvr, r_idx, r_cache, G, bias=None):
+        args, out, _keep = self._args(l_bvr, l_idx, l_cache, r_bvr, r_idx, r_cache, G, bias)
+        rc = self.lib.sbvr_port_mm_T_v1(*args)
+        if rc != 0:
+            raise RuntimeError(f"sbvr_port_mm_T_v1 failed: {rc}")
+        return out
+
+    def time_mm_T_v1(self, l_bvr, l_idx, l_cache, r_bvr, r_idx, r_cache, G, bias=None, warmup=10, iters=100):
+        """Mean seconds per call, timed inside the library."""
+        args, _out, _keep = self._args(l_bvr, l_idx, l_cache, r_bvr, r_idx, r_cache, G, bias)
+        t = self.lib.sbvr_port_time_mm_T_v1(*args, int(warmup), int(iters))
+        if t < 0:
+            raise RuntimeError("sbvr_port_time_mm_T_v1 failed")
+        return t
+
+
+PORT = _Port()

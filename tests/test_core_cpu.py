@@ -1,0 +1,178 @@
+"""Host-side package tests (no GPU): the sbvr objects, their layouts, decode(),
+save/load and the encoder, against the golden vectors the reference wrote."""
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GOLDEN, ROOT
+
+CASES = {
+    "default_s2": {}, "default_s3": {}, "pad_s2": {}, "v2_s2": {"cpu_kernel_v2": True},
+    "trans_s2": {"trans": True}, "v1_s2": {"cpu_kernel": True}, "v1_row_s2": {"cpu_kernel": True},
+}
+
+
+def _t(a):
+    return torch.from_numpy(np.ascontiguousarray(a))
+
+
+def _same_bits(a, b):
+    return a.shape == b.shape and torch.equal(a.contiguous().view(torch.uint8), b.contiguous().view(torch.uint8))
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_encoder_reproduces_reference(golden, name):
+    """Same input, same configuration, CPU: identical bvr, coeff_idx and coeff_cache."""
+    import sbvr
+    g = golden(name)
+    obj = sbvr.sbvr(_t(g["data"]), encoder_config={"num_sums": int(g["num_sums"])},
+                    device=torch.device("cpu"), verbose_level=0, **CASES[name])
+    assert _same_bits(obj.bvr.data, _t(g["bvr"]))
+    assert _same_bits(obj.coeff_idx.data, _t(g["coeff_idx"]))
+    assert _same_bits(obj.coeff_cache.data, _t(g["coeff_cache"]))
+    if g["decoded"].size:
+        assert _same_bits(obj.decode(), _t(g["decoded"]))
+
+
+@pytest.mark.parametrize("name", ["default_s2", "default_s3", "default_s4", "pad_s2", "v2_s2", "v1_row_s2",
+                                  "trans_s2", "weights_s4"])
+def test_decode_of_reference_arrays(golden, name):
+    import sbvr
+    g = golden(name)
+    obj = sbvr.sbvr.from_parts(_t(g["bvr"]), _t(g["coeff_idx"]), _t(g["coeff_cache"]), int(g["bvr_len"]),
+                               original_shape=g["decoded"].shape)
+    assert _same_bits(obj.decode(), _t(g["decoded"]))
+
+
+def test_load_file_written_by_reference(golden):
+    """default_s2_saved.pt was written by the reference's save(); the class path in
+    the pickle is sbvr.core._sbvr_serialized."""
+    import sbvr
+    obj = sbvr.load(os.path.join(GOLDEN, "default_s2_saved.pt"), device="cpu", verbose_level=0)
+    g = golden("default_s2")
+    assert _same_bits(obj.bvr.data, _t(g["bvr"])) and _same_bits(obj.decode(), _t(g["decoded"]))
+    assert obj.num_sums == 2 and obj.bvr_len == 256
+
+
+def test_save_load_round_trip(tmp_path, golden):
+    import sbvr
+    g = golden("weights_s4")
+    obj = sbvr.sbvr.from_parts(_t(g["bvr"]), _t(g["coeff_idx"]), _t(g["coeff_cache"]), 256)
+    path = str(tmp_path / "w.pt")
+    obj.save(path)
+    back = sbvr.load(path, device="cpu", verbose_level=0)
+    assert _same_bits(back.bvr.data, obj.bvr.data) and _same_bits(back.coeff_idx.data, obj.coeff_idx.data)
+    assert _same_bits(back.coeff_cache.data, obj.coeff_cache.data)
+    assert _same_bits(back.decode(), obj.decode())
+    with pytest.raises(ValueError):
+        sbvr.load(path, device="cpu", verbose_level=0, cpu_kernel_v2=True)     # uint32 file, uint8 requested
+
+
+def test_layout_conversions(golden):
+    """uint32 <-> uint8 re-wording and the 16-lane layout are pure permutations."""
+    from sbvr import layout
+    g = golden("default_s4")
+    bvr = _t(g["bvr"])
+    sel = layout.default_to_sel(bvr)
+    b8 = layout.rewidth(bvr, torch.uint8)
+    assert b8.shape == (bvr.shape[0] * 4, bvr.shape[1], bvr.shape[2])
+    assert torch.equal(layout.default_to_sel(b8), sel)
+    assert _same_bits(layout.rewidth(b8, torch.uint32), bvr)
+    g1 = golden("v1_s2")
+    v1 = _t(g1["bvr"])
+    planes = layout.v1_to_planes(v1)
+    assert _same_bits(layout.planes_to_v1(planes.reshape(planes.shape[0], -1), planes.shape[1]), v1)
+    v2 = _t(golden("v2_s2")["bvr"])
+    assert _same_bits(layout.planes_to_default(layout.default_to_planes(v2).reshape(v2.shape[2], -1), v2.shape[1]), v2)
+
+
+def test_group_length_128_extension():
+    """bvr_len is a parameter here (the reference fixes 256): encode, decode, error band."""
+    import sbvr
+    torch.manual_seed(0)
+    w = (torch.randn(4, 256) * 0.02).to(torch.float16)
+    obj = sbvr.sbvr(w, encoder_config={"num_sums": 4, "bvr_len": 128}, device=torch.device("cpu"), verbose_level=0)
+    assert obj.bvr.shape == (8, 4, 4) and obj.coeff_idx.shape == (2, 4) and obj.bvr.dtype == torch.uint32
+    rel = ((obj.decode().float() - w.float()) ** 2).mean() / w.float().var()
+    assert rel < 0.03          # the reference logs about 1.7e-2 of the variance for 4 planes (test.txt:55-59)
+
+
+def test_constructor_errors():
+    import sbvr
+    with pytest.raises(ValueError):
+        sbvr.sbvr()
+    with pytest.raises(ValueError):
+        sbvr.sbvr(torch.zeros(2, 256), sbvr_serialized=object())
+    with pytest.raises(ValueError):
+        sbvr.sbvr(sbvr_serialized=object())
+    with pytest.raises(ValueError):
+        sbvr.sbvr(torch.zeros(2, 256), encoder_config={"bvr_len": 48}, device="cpu", verbose_level=0)
+
+
+def test_synthetic_encoding_shapes():
+    from sbvr import synth
+    bvr, idx, cache = synth.random_encoding(64, 512, 3, 128, 300, seed=1)
+    assert bvr.shape == (16, 64, 3) and bvr.dtype == torch.uint32
+    assert idx.shape == (4, 64) and idx.dtype == torch.uint16 and int(idx.to(torch.int32).max()) < 300
+    assert cache.shape == (300, 3) and cache.dtype == torch.float16
+    assert torch.all(cache.float().abs()[:, :-1] <= cache.float().abs()[:, 1:])     # sorted by magnitude
+
+
+def test_ops_refuse_cpu_tensors():
+    """No CPU fallback: the operators raise on host tensors."""
+    import sbvr
+    from sbvr import synth
+    bvr, idx, cache = synth.random_encoding(32, 256, 4, 128, 16)
+    x = torch.zeros((1, 256), dtype=torch.float16)
+    with pytest.raises(sbvr.SbvrHipError):
+        sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, 128)
+
+
+# ------------------------------------------------------------------ C ABI
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sbvr_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sbvr_hip_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    """libsbvr_hip.so loads without a GPU and exports what include/sbvr_hip.h declares."""
+    import ctypes
+    from sbvr import hip
+    path = hip.library_path()
+    assert os.path.exists(path), f"{path} missing: run __graft_entry__.build()"
+    lib = ctypes.CDLL(path)
+    names = _declared_symbols()
+    assert len(names) >= 7
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in sbvr_hip.h but not exported"
+    lib.sbvr_hip_version.restype = ctypes.c_int
+    assert lib.sbvr_hip_version() == 100
+    lib.sbvr_hip_linear_f16_workspace.restype = ctypes.c_size_t
+    assert lib.sbvr_hip_linear_f16_workspace(1, 14336, 4096, 4, 128) == 14336 * 8
+    assert lib.sbvr_hip_linear_f16_workspace(1, 64, 96, 4, 32) == 0        # portable kernel: no workspace
+
+
+def test_argument_validation_without_gpu():
+    """Bad arguments are rejected before anything touches a device."""
+    import ctypes
+    from sbvr import hip
+    lib = hip._load()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    rc = lib.sbvr_hip_linear_f16(None, p, p, 1, p, None, p, 1, 16, 128, 4, 128, 4, None, 0, 0, None)
+    assert rc == -1 and b"null" in lib.sbvr_hip_last_error()
+    rc = lib.sbvr_hip_linear_f16(p, p, p, 1, p, None, p, 1, 16, 100, 4, 128, 4, None, 0, 0, None)
+    assert rc == -1 and b"multiple" in lib.sbvr_hip_last_error()
+    rc = lib.sbvr_hip_linear_f16(p, p, p, 3, p, None, p, 1, 16, 128, 4, 128, 4, None, 0, 0, None)
+    assert rc == -1 and b"idx_bytes" in lib.sbvr_hip_last_error()
+    rc = lib.sbvr_hip_linear_f16(p, p, p, 1, p, None, p, 1, 16, 128, 4, 128, 300, None, 0, 0, None)
+    assert rc == -1 and b"uint8" in lib.sbvr_hip_last_error()
+    rc = lib.sbvr_hip_mm_T(p, p, 1, p, p, p, 1, p, None, p, 1, 16, 100, 4, 4, 128, 4, 4, None)
+    assert rc == -1
+    rc = lib.sbvr_hip_row_deq_mm_T(p, p, p, 1, p, None, p, 1, 48, 64, 4, 32, 4, None)
+    assert rc == -1        # N must be a multiple of 32 and of G

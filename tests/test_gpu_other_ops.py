@@ -1,0 +1,127 @@
+"""GPU parity of the reference-compatible alternates (both-encoded _sbvr_mm_T and
+the trans=True _sbvr_row_deq_mm_T) and of SBVRLinear, against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand_enc(rng, rows, K, S, G, L, oracle):
+    sel = rng.integers(0, 1 << S, size=rows * K).astype(np.int32)
+    bvr = oracle.C.planes_to_default(oracle.C.sel_to_planes(sel, S, 32), rows, K)
+    idx = rng.integers(0, L, size=(K // G, rows)).astype(np.uint8 if L <= 256 else np.uint16)
+    cache = (rng.standard_normal((L, S)) * 0.5).astype(np.float16)
+    return bvr, idx, cache
+
+
+def _close(y, yd, ulps=2.0):
+    got = y.float().cpu().numpy().astype(np.float64)
+    rms = float(np.sqrt(np.mean(yd ** 2))) + 1e-30
+    assert (np.abs(got - yd) / np.maximum(np.abs(yd), 1e-2 * rms)).max() <= 1e-2
+    assert (np.abs(got - yd) / (np.maximum(np.abs(yd), rms) * 2.0 ** -10)).max() <= ulps
+
+
+@pytest.mark.parametrize("M,N,K,Sl,Sr,G,Ll,Lr", [(1, 64, 512, 4, 4, 256, 5, 9), (3, 40, 256, 2, 3, 128, 300, 7),
+                                                 (2, 33, 512, 8, 6, 256, 4, 400)])
+def test_mm_T(oracle, M, N, K, Sl, Sr, G, Ll, Lr):
+    import sbvr
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(M * 100 + N)
+    lb, li, lc = _rand_enc(rng, M, K, Sl, G, Ll, oracle)
+    rb, ri, rc = _rand_enc(rng, N, K, Sr, G, Lr, oracle)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    y = sbvr._sbvr_mm_T(t(lb), t(li), t(lc), t(rb), t(ri), t(rc), torch.zeros(0, dtype=torch.float16, device=dev),
+                        bvr_len=G)
+    _, yd = oracle.C.mm_T(lb, li, lc, rb, ri, rc, G)
+    _close(y, yd)
+    bias = (rng.standard_normal(N)).astype(np.float16)
+    yb = sbvr._sbvr_mm_T(t(lb), t(li), t(lc), t(rb), t(ri), t(rc), t(bias), bvr_len=G)
+    want, _ = oracle.C.mm_T(lb, li, lc, rb, ri, rc, G, bias)
+    d = np.abs(yb.float().cpu().numpy().astype(np.float64) - want.astype(np.float64))
+    assert d.max() <= 2.0 ** -9 * max(np.abs(want.astype(np.float64)).max(), 1.0)
+
+
+def test_mm_T_object_api(oracle, golden):
+    """sbvr.mm_T(lhs, rhs, bias) on objects built from the reference's encodings."""
+    import sbvr
+    dev = torch.device("cuda:0")
+    g = golden("default_s2")
+    mk = lambda: sbvr.sbvr.from_parts(*(torch.from_numpy(g[k]).to(dev) for k in ("bvr", "coeff_idx", "coeff_cache")), 256)
+    a, b = mk(), mk()
+    y = sbvr.mm_T(a, b, None)
+    _, yd = oracle.C.mm_T(g["bvr"], g["coeff_idx"], g["coeff_cache"], g["bvr"], g["coeff_idx"], g["coeff_cache"], 256)
+    _close(y, yd)
+    w = g["decoded"].astype(np.float64)
+    assert np.abs(y.float().cpu().numpy() - w @ w.T).max() <= 1e-2 * np.abs(w @ w.T).max()
+
+
+@pytest.mark.parametrize("M,N,K,S,G,L", [(1, 256, 64, 4, 256, 9), (2, 512, 40, 2, 128, 300)])
+def test_row_deq_mm_T(oracle, M, N, K, S, G, L):
+    import sbvr
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(N + K)
+    # the encoded tensor is W^T: K rows of N columns, groups along N
+    bvr, idx, cache = _rand_enc(rng, K, N, S, G, L, oracle)         # (N/32, K, S), (N/G, K)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    y = sbvr._sbvr_row_deq_mm_T(t(x), t(bvr), t(idx), t(cache), t(bias), 0, bvr_len=G)
+    want = oracle.C.row_deq_mm_T(x, bvr, idx, cache, G, bias).astype(np.float64)
+    d = np.abs(y.float().cpu().numpy().astype(np.float64) - want)
+    assert d.max() <= 2.0 ** -9 * max(np.abs(want).max(), 1.0)
+
+
+def test_row_deq_golden(oracle, golden):
+    import sbvr
+    dev = torch.device("cuda:0")
+    g = golden("trans_s2")
+    K, N = g["decoded"].shape
+    x = torch.randn((2, K), generator=torch.Generator().manual_seed(3)).to(torch.float16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    y = sbvr._sbvr_row_deq_mm_T(x.to(dev), t(g["bvr"]), t(g["coeff_idx"]), t(g["coeff_cache"]),
+                                torch.zeros(0, dtype=torch.float16, device=dev), 0)
+    want = x.numpy().astype(np.float64) @ g["decoded"].astype(np.float64)
+    assert np.abs(y.float().cpu().numpy() - want).max() <= 1e-2 * np.abs(want).max()
+
+
+def test_sbvr_linear_module(oracle, golden):
+    """SBVRLinear on a reference encoding: leading dims, padding of K, bias, > 16 rows."""
+    import sbvr
+    dev = torch.device("cuda:0")
+    g = golden("pad_s2")                       # weight (3, 300) padded to 512
+    enc = sbvr.sbvr.from_parts(*(torch.from_numpy(g[k]).to(dev) for k in ("bvr", "coeff_idx", "coeff_cache")), 256,
+                               original_shape=(3, 300))
+    lin = sbvr.SBVRLinear.from_sbvr(enc)
+    x = torch.randn((2, 5, 300), generator=torch.Generator().manual_seed(4)).to(torch.float16)
+    y = lin(x.to(dev))
+    assert y.shape == (2, 5, 3)
+    want = x.numpy().astype(np.float64) @ g["decoded"].astype(np.float64).T
+    assert np.abs(y.float().cpu().numpy() - want).max() <= 1e-2 * np.abs(want).max()
+    from sbvr import synth
+    bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(128, 256, 4, 128, 64, seed=2))
+    bias = torch.randn(128, generator=torch.Generator().manual_seed(5)).to(torch.float16)
+    lin2 = sbvr.SBVRLinear(256, 128, bvr, idx, cache, 128, bias.to(dev))
+    x2 = torch.randn((40, 256), generator=torch.Generator().manual_seed(6)).to(torch.float16)
+    y2 = lin2(x2.to(dev))
+    yref, _ = oracle.C.linear_f16(x2.numpy(), bvr.cpu().numpy(), idx.cpu().numpy(), cache.cpu().numpy(), 128, bias.numpy())
+    d = np.abs(y2.float().cpu().numpy().astype(np.float64) - yref.astype(np.float64))
+    assert d.max() <= 2.0 ** -9 * np.abs(yref.astype(np.float64)).max()
+
+
+def test_hip_init_and_bad_arguments():
+    import sbvr
+    dev = torch.device("cuda:0")
+    sbvr._sbvr_hip_init(dev)
+    from sbvr import synth
+    bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(32, 256, 4, 128, 16))
+    x = torch.zeros((1, 256), dtype=torch.float16, device=dev)
+    with pytest.raises(TypeError):
+        sbvr._sbvr_linear_f16(x.float(), bvr, idx, cache, None, 128)
+    with pytest.raises(ValueError):
+        sbvr._sbvr_linear_f16(x[:, :128], bvr, idx, cache, None, 128)
+    with pytest.raises(ValueError):
+        sbvr._sbvr_linear_f16(torch.zeros((2, 512), dtype=torch.float16, device=dev)[:, ::2],
+                              bvr, idx, cache, None, 128)                                  # not contiguous
+    with pytest.raises(TypeError):
+        sbvr._sbvr_linear_f16(x, bvr, idx.to(torch.uint16), cache, None, 128)          # 16 lines want uint8
