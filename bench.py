@@ -28,6 +28,9 @@ sys.path.insert(0, ROOT)
 N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH = 14336, 4096, 4, 128, 256, 1
 COPIES = 16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the gate GEMV, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
+# 256 MiB copy (profiles/sbvr_gemv_mfma_gate_4096x14336.txt): 30.08 MB read + 1.06 MB written.
+MEASURED_TRAFFIC_BYTES = 31.14e6
 
 
 def algorithmic_bytes(n, k, s, g, lines, m):
@@ -143,10 +146,19 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy, the known-size kernel that "
+                         "hardware byte counters are scaled by when profiling")
     a = ap.parse_args()
     if a.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the path is single-GPU in this build (run with --gpus 1)")
 
+    if a.calibrate_copy:
+        import torch
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
     wall_ms, event_ms, launcher, device = gpu_leg(a.steps, a.warmup)
     nbytes = algorithmic_bytes(N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH)
     value = nbytes / (wall_ms * 1e-3) / 1e9
@@ -181,7 +193,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "us_per_launch": round(event_ms * 1e3, 3),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES,
         },
     }
     if not a.no_cpu:
