@@ -126,6 +126,16 @@ constexpr int kWavesPerWG = 4;
 constexpr int kThreads = 64 * kWavesPerWG;
 constexpr int kMaxM = 16;        // batch rows of the decode kernel (row tiles of 4)
 constexpr float kLastTermScale = 256.f;  // third fp8 term of an activation holds residual * 256
+#ifndef SBVR_PREFETCH
+#define SBVR_PREFETCH 8
+#endif
+#ifndef SBVR_HEAD
+#define SBVR_HEAD 0
+#endif
+#ifndef SBVR_STREAM_AFTER_PREP
+#define SBVR_STREAM_AFTER_PREP 0
+#endif
+constexpr int kPrefetch = SBVR_PREFETCH;  // units requested ahead of the one being consumed
 constexpr int kTableRegs = 4;             // uint4 per thread while the coefficient table is staged
 constexpr size_t kMaxTableLds = kTableRegs * 16 * 256;   // largest coefficient table staged in LDS (16 KB)
 
@@ -147,6 +157,7 @@ struct GemvArgs {
     uint16_t *out;
     unsigned long long *acc;   // (M, N) split-K accumulators, all zero between calls
     int M, N, K, G, L;
+    int gshift;           // a coefficient group is 128 << gshift elements
     int n_tiles;          // workgroups along N
     int ksplit;           // workgroups along K
 #ifdef SBVR_TRACE
@@ -160,7 +171,7 @@ __host__ __device__ constexpr size_t align16(size_t v) { return (v + 15) & ~stat
 #define SBVR_STAMP(i)                                                         \
     do {                                                                      \
         if (a.trace && threadIdx.x == 0)                                      \
-            a.trace[blockIdx.x * 8 + (i)] = wall_clock64();                   \
+            a.trace[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = wall_clock64();                   \
     } while (0)
 unsigned long long *g_trace = nullptr;
 #else
@@ -256,7 +267,8 @@ __device__ __forceinline__ void load_coeffs(P cache, int line, float (&c)[S])
 constexpr int gemv_waves(int S, int MT, int CT, int SP)
 {
     // queued units, double-buffered products, A operands, sums, coefficients, scratch
-    const int regs = CT * SP * (S + 1) + 8 * MT * S + 8 * MT + CT * MT + S + (S < 4 ? 20 : 4);
+    const int live = CT * SP < kPrefetch + 1 ? CT * SP : kPrefetch + 1;
+    const int regs = live * (S + 1) + 8 * MT * S + 8 * MT + CT * MT + S + (S < 4 ? 28 : 12);
     const int w = 512 / regs;
     return w < 1 ? 1 : (w > 8 ? 8 : w);
 }
@@ -306,13 +318,12 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int nt = blockIdx.x % a.n_tiles;
-    const int kp = blockIdx.x / a.n_tiles;
+    const int nt = blockIdx.x;   // workgroup along N
+    const int kp = blockIdx.y;   // workgroup along K
     const int N = a.N, K = a.K;
     const int col = lane & 15;   // column inside a tile (B and D operands)
     const int blk = lane >> 4;   // word of the sub-group (B), batch row of the tile (D)
     const int sg0 = kp * SP;     // first sub-group of this workgroup
-    const int gsub = a.G / kSub; // sub-groups per coefficient group
     // The wave owns columns [n_own, n_own + 16*CT).  It computes a full window
     // of 16*CT columns; a window that would stick out of N is moved left, and
     // the columns it then shares with its neighbour are left to the neighbour.
@@ -320,20 +331,45 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     const int n_base = min(n_own, N - CT * 16);
 
     SBVR_STAMP(0);
-    // -- 1. clear the A images, then issue every global load of the wave, oldest
-    //       first: the activations of its share of the A images, its slice of the
-    //       coefficient table, then the whole weight stream.  Waiting for an early
-    //       load never drains the later ones.
-    for (int i = tid; i < SP * MT * 512; i += kThreads)
-        reinterpret_cast<uint32_t *>(img)[i] = 0u;
+    // -- 1. The vector-memory queue of a CU holds only a few tens of KB; a wave
+    //       that issues more stalls at the load until there is room.  So the
+    //       stream is started with the first kAhead units only, the small loads
+    //       every wave needs before its first MFMA (activations, table slice)
+    //       follow right behind them, and each later unit is requested kAhead
+    //       units before it is consumed.  Unit u = (sub-group u / CT, tile u % CT).
+    constexpr int U = SP * CT;
+    constexpr int kAhead = U < kPrefetch ? U : kPrefetch;
+    Planes<S> q[U];
+    int qline[U];
+    const uint32_t lane_w = (static_cast<uint32_t>(blk) * N + n_base + col) * S;   // words
+    const uint32_t lane_i = static_cast<uint32_t>(n_base + col);
+    auto request = [&](int u) {
+        const int sgi = u / CT, ct = u % CT;
+        const uint32_t *wrow = a.bvr + static_cast<size_t>(sg0 + sgi) * 4 * N * S;     // wave-uniform
+        const IdxT *irow = static_cast<const IdxT *>(a.idx) + static_cast<size_t>((sg0 + sgi) >> a.gshift) * N;
+        q[u] = load_planes<S>(wrow + lane_w + ct * 16 * S);
+#ifdef SBVR_HACK_NOIDX
+        qline[u] = (lane + u) & 255; (void)irow;
+#else
+        qline[u] = static_cast<int>(irow[lane_i + ct * 16]);
+#endif
+    };
+    constexpr int kHead = kAhead < SBVR_HEAD ? kAhead : SBVR_HEAD;   // units requested before the small loads
+#pragma unroll
+    for (int u = 0; u < kHead; ++u)
+        request(u);
     constexpr int kTasks = SP * MT;          // image tasks per wave, at most (M <= 4*MT)
     uint32_t xx[kTasks];
 #pragma unroll
     for (int t = 0; t < kTasks; ++t) {
         const int task = wave + kWavesPerWG * t;     // task = m * SP + sgi
         const int m = task / SP, sgi = task % SP;
+#ifdef SBVR_HACK_NOPROLOGUE
+        xx[t] = lane * 77u + m; (void)sgi;
+#else
         xx[t] = *reinterpret_cast<const uint32_t *>(
             a.x + (m < a.M ? static_cast<size_t>(m) * K + static_cast<size_t>(sg0 + sgi) * kSub + 2 * lane : 0));
+#endif
     }
     uint4 treg[kTableRegs];
     const int tvecs = a.L * S / 8;           // the table is a whole number of 16-byte vectors here
@@ -341,26 +377,16 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
         for (int r = 0; r < kTableRegs; ++r) {
             const int i = tid + r * kThreads;
-            treg[r] = reinterpret_cast<const uint4 *>(a.cache)[i < tvecs ? i : 0];
+#ifdef SBVR_HACK_NOPROLOGUE
+            treg[r] = uint4{1u, 2u, 3u, 4u};
+#else
+            if (r * kThreads < tvecs)        // wave-uniform: small tables take one pass
+                treg[r] = reinterpret_cast<const uint4 *>(a.cache)[i < tvecs ? i : 0];
+#endif
         }
     }
-
-    Planes<S> q[SP][CT];
-    int qline[SP][CT];
-    {
-        const uint32_t lane_w = (static_cast<uint32_t>(blk) * N + n_base + col) * S;   // words
-        const uint32_t lane_i = static_cast<uint32_t>(n_base + col);
-#pragma unroll
-        for (int sgi = 0; sgi < SP; ++sgi) {
-            const uint32_t *wrow = a.bvr + static_cast<size_t>(sg0 + sgi) * 4 * N * S;     // wave-uniform
-            const IdxT *irow = static_cast<const IdxT *>(a.idx) + static_cast<size_t>((sg0 + sgi) / gsub) * N;
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) {
-                q[sgi][ct] = load_planes<S>(wrow + lane_w + ct * 16 * S);
-                qline[sgi][ct] = static_cast<int>(irow[lane_i + ct * 16]);
-            }
-        }
-    }
+    for (int i = tid; i < SP * MT * 512; i += kThreads)
+        reinterpret_cast<uint32_t *>(img)[i] = 0u;
     if constexpr (TBL) {
 #pragma unroll
         for (int r = 0; r < kTableRegs; ++r) {
@@ -383,7 +409,11 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
         for (int t = 0; t < kTasks; ++t) {
             const int task = wave + kWavesPerWG * t;
             const int m = task / SP, sgi = task % SP;
+#ifdef SBVR_HACK_NOPREP
+            if (m < a.M && a.L < 0) {
+#else
             if (m < a.M) {
+#endif
                 // 2^e puts the largest magnitude of the sub-group into [32, 64)
                 // (fp16 bits order like magnitudes; subnormals count as 2^-15)
                 const uint32_t amax = wave_umax(max(xx[t] & 0x7fffu, (xx[t] >> 16) & 0x7fffu));
@@ -412,8 +442,18 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
             }
         }
     }
+#if SBVR_STREAM_AFTER_PREP == 0
+#pragma unroll
+    for (int u = kHead; u < kAhead; ++u)
+        request(u);
+#endif
     __syncthreads();
     SBVR_STAMP(3);
+#if SBVR_STREAM_AFTER_PREP == 1
+#pragma unroll
+    for (int u = kHead; u < kAhead; ++u)
+        request(u);
+#endif
 
     // -- 3. consume the units: sub-group outer (A operand stays in registers),
     //       column tile inner.  The MFMAs of a unit are issued before the
@@ -430,8 +470,8 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     v4f D[2][MT][S];
     float cprev[S];
     float scprev[MT];
-    auto products = [&](int sgi, int ct, v4f (&Dn)[MT][S]) {
-        const Planes<S> &pl = q[sgi][ct];
+    auto products = [&](int u, v4f (&Dn)[MT][S]) {
+        const Planes<S> &pl = q[u];
 #pragma unroll
         for (int j = 0; j < S; ++j) {
             const uint32_t w = pl.w[j];
@@ -448,8 +488,8 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
             }
         }
     };
-    auto coeffs_of = [&](int sgi, int ct, float (&c)[S]) {
-        const int line = min(qline[sgi][ct], a.L - 1);
+    auto coeffs_of = [&](int u, float (&c)[S]) {
+        const int line = min(qline[u], a.L - 1);
         if constexpr (TBL)
             load_coeffs<S>(static_cast<const uint16_t *>(table), line, c);
         else
@@ -476,9 +516,11 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
                 sc[mt] = scales[sgi * (MT * 4) + mt * 4 + blk];
             }
         }
+        if (u + kAhead < U)
+            request(u + kAhead);
         float c[S];
-        coeffs_of(sgi, ct, c);
-        products(sgi, ct, D[u & 1]);
+        coeffs_of(u, c);
+        products(u, D[u & 1]);
         if (u > 0)
             fold((u - 1) % CT, D[(u - 1) & 1]);
 #pragma unroll
@@ -492,56 +534,65 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     fold((SP * CT - 1) % CT, D[(SP * CT - 1) & 1]);
 
     SBVR_STAMP(4);
-    // -- 4. results: direct when K is not split, else through the accumulators
+#ifdef SBVR_HACK_NOFINAL
+    { float t = 0.f; for (int ct = 0; ct < CT; ++ct) for (int mt = 0; mt < MT; ++mt) t += y[ct][mt]; if (t == 123.456f) a.out[0] = 1; return; }
+#endif
+    // -- 4. results: direct when K is not split, else through the accumulators.
+    //       A lane holds column n_base + 16*ct + col of batch row 4*mt + blk.
+    const bool shifted = n_base != n_own;            // wave-uniform: window moved left at the edge of N
+    bool valid[CT][MT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            valid[ct][mt] = (mt * 4 + blk < a.M) && (!shifted || n_base + ct * 16 + col >= n_own);
+    const size_t lane_o = static_cast<size_t>(blk) * N + n_base + col;
+    uint16_t *outp = a.out + lane_o;
+    auto store = [&](int ct, int mt, float v) {
+        uint16_t r = f2h(v);
+        if (a.bias)
+            r = hadd(r, a.bias[n_base + ct * 16 + col]);
+        outp[static_cast<size_t>(mt) * 4 * N + ct * 16] = r;
+    };
     if (a.ksplit == 1) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            const int n = n_base + ct * 16 + col;
+        for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int m = mt * 4 + blk;
-                if (n >= n_own && m < a.M) {
-                    uint16_t r = f2h(y[ct][mt]);
-                    if (a.bias)
-                        r = hadd(r, a.bias[n]);
-                    a.out[static_cast<size_t>(m) * N + n] = r;
-                }
-            }
-        }
+            for (int mt = 0; mt < MT; ++mt)
+                if (valid[ct][mt])
+                    store(ct, mt, y[ct][mt]);
         return;
     }
-    unsigned long long old[CT][MT], adds[CT][MT];
+    unsigned long long *accp = a.acc + lane_o;
+    unsigned long long tot[CT][MT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
-        const int n = n_base + ct * 16 + col;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            const int m = mt * 4 + blk;
-            old[ct][mt] = 0ull;
-            adds[ct][mt] = (1ull << 56) + static_cast<unsigned long long>(to_fixed(y[ct][mt]) + kAccBias);
-            if (n >= n_own && m < a.M)
-                old[ct][mt] = __hip_atomic_fetch_add(&a.acc[static_cast<size_t>(m) * N + n], adds[ct][mt],
-                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            tot[ct][mt] = (1ull << 56) + static_cast<unsigned long long>(to_fixed(y[ct][mt]) + kAccBias);
+            unsigned long long old = 0ull;
+            if (valid[ct][mt])
+                old = __hip_atomic_fetch_add(accp + static_cast<size_t>(mt) * 4 * N + ct * 16, tot[ct][mt],
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            tot[ct][mt] += old;
         }
     }
     SBVR_STAMP(5);
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
-        const int n = n_base + ct * 16 + col;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            const int m = mt * 4 + blk;
-            const unsigned long long tot = old[ct][mt] + adds[ct][mt];
-            if (n >= n_own && m < a.M && static_cast<int>(tot >> 56) == a.ksplit) {
-                const long long sum = static_cast<long long>(tot & ((1ull << 56) - 1)) -
-                                      static_cast<long long>(a.ksplit) * kAccBias;
-                const float total = static_cast<float>(static_cast<double>(sum) * (1.0 / (1 << kAccFracBits)));
-                __hip_atomic_store(&a.acc[static_cast<size_t>(m) * N + n], 0ull,
+            if (valid[ct][mt] && static_cast<int>(tot[ct][mt] >> 56) == a.ksplit) {
+                // the sum without the count and the ksplit biases, back to float:
+                // sum = hi * 2^24 + lo, both halves exact in fp32, one rounding
+                const long long sum = static_cast<long long>(tot[ct][mt] & ((1ull << 56) - 1)) -
+                                      (static_cast<long long>(a.ksplit) << 47);
+                const float hi = static_cast<float>(static_cast<int>(sum >> 24));
+                const float lo = static_cast<float>(static_cast<int>(sum & 0xffffff));
+                const float total = fmaf(hi, 1.f / (1 << (kAccFracBits - 24)), lo * (1.f / (1 << kAccFracBits)));
+                __hip_atomic_store(accp + static_cast<size_t>(mt) * 4 * N + ct * 16, 0ull,
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                uint16_t r = f2h(total);
-                if (a.bias)
-                    r = hadd(r, a.bias[n]);
-                a.out[static_cast<size_t>(m) * N + n] = r;
+                store(ct, mt, total);
             }
         }
     }
@@ -561,7 +612,7 @@ int env_int(const char *name, int dflt)
 }
 
 // (CT, SP) pairs that have a kernel instance; see the dispatch below.
-constexpr int kShapes[][2] = {{1, 1}, {2, 1}, {4, 1}, {8, 1}, {2, 2}, {4, 2}, {8, 2}, {2, 4}, {4, 4}, {1, 8}, {2, 8}};
+constexpr int kShapes[][2] = {{1, 1}, {2, 1}, {4, 1}, {8, 1}, {2, 2}, {4, 2}, {8, 2}, {2, 4}, {4, 4}, {1, 8}, {2, 8}, {4, 8}, {8, 4}};
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
 
 bool shape_ok_for(int MT, int CT, int SP)
@@ -620,7 +671,7 @@ GemvPlan plan_gemv(int M, int N, int K, int S, int L, int idx_bytes, int cus)
 bool mfma_path_ok(int M, int N, int K, int S, int G)
 {
     // 32-bit element offsets into bvr
-    return M >= 1 && M <= kMaxM && N >= 16 && K % kSub == 0 && G % kSub == 0 &&
+    return M >= 1 && M <= kMaxM && N >= 16 && K % kSub == 0 && G % kSub == 0 && ((G / kSub) & (G / kSub - 1)) == 0 &&
            (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) &&
            static_cast<double>(K / 32) * N * S < 2147483648.0 && K / kSub <= kMaxKsplit;
 }
@@ -628,13 +679,15 @@ bool mfma_path_ok(int M, int N, int K, int S, int G)
 template <int S, int MT, int CT, int SP>
 hipError_t launch_gemv_inst(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
-    const dim3 grid(static_cast<unsigned>(p.n_tiles) * p.ksplit), block(kThreads);
+    const dim3 grid(static_cast<unsigned>(p.n_tiles), static_cast<unsigned>(p.ksplit)), block(kThreads);
     if (p.mode == 0)
         hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, 0>), grid, block, p.lds, st, a);
+#ifndef SBVR_FAST_BUILD
     else if (p.mode == 1)
         hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, 1>), grid, block, p.lds, st, a);
     else
         hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, 2>), grid, block, p.lds, st, a);
+#endif
     return hipGetLastError();
 }
 
@@ -647,7 +700,7 @@ hipError_t launch_gemv_shape(const GemvArgs &a, const GemvPlan &p, hipStream_t s
     SBVR_SHAPE(1, 1); SBVR_SHAPE(2, 1); SBVR_SHAPE(4, 1); SBVR_SHAPE(8, 1);
     SBVR_SHAPE(2, 2); SBVR_SHAPE(4, 2); SBVR_SHAPE(2, 4); SBVR_SHAPE(1, 8);
     if constexpr (MT == 1) {
-        SBVR_SHAPE(8, 2); SBVR_SHAPE(4, 4); SBVR_SHAPE(2, 8);
+        SBVR_SHAPE(8, 2); SBVR_SHAPE(4, 4); SBVR_SHAPE(2, 8); SBVR_SHAPE(4, 8); SBVR_SHAPE(8, 4);
     }
 #undef SBVR_SHAPE
     return hipErrorInvalidConfiguration;
@@ -665,6 +718,11 @@ hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 
 hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
+#ifdef SBVR_FAST_BUILD      // development builds: one instantiation family only
+    if (S == 4 && p.MT == 1 && p.mode == 0)
+        return launch_gemv_shape<4, 1>(a, p, st);
+    return hipErrorInvalidConfiguration;
+#else
     switch (S) {
     case 2: return launch_gemv_mt<2>(a, p, st);
     case 3: return launch_gemv_mt<3>(a, p, st);
@@ -672,6 +730,7 @@ hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t 
     case 6: return launch_gemv_mt<6>(a, p, st);
     default: return launch_gemv_mt<8>(a, p, st);
     }
+#endif
 }
 
 int current_cus()
@@ -827,6 +886,7 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
         a.bias = static_cast<const uint16_t *>(bias);
         a.out = static_cast<uint16_t *>(out);
         a.M = M; a.N = N; a.K = K; a.G = G; a.L = L;
+        a.gshift = __builtin_ctz(static_cast<unsigned>(G / kSub));
         a.n_tiles = p.n_tiles; a.ksplit = p.ksplit;
 #ifdef SBVR_TRACE
         a.trace = g_trace;
