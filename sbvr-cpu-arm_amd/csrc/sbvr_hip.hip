@@ -122,22 +122,9 @@ sbvr_linear_portable_kernel(const uint16_t *__restrict__ x, const uint32_t *__re
 // --------------------------------------------------------------- MFMA decode
 
 constexpr int kSub = 128;        // K elements per MFMA (one sub-group)
-constexpr int kWavesPerWG = 4;
-constexpr int kThreads = 64 * kWavesPerWG;
+constexpr int kMaxWaves = 16;    // waves of a workgroup; they split K among themselves
 constexpr int kMaxM = 16;        // batch rows of the decode kernel (row tiles of 4)
 constexpr float kLastTermScale = 256.f;  // third fp8 term of an activation holds residual * 256
-#ifndef SBVR_PREFETCH
-#define SBVR_PREFETCH 8
-#endif
-#ifndef SBVR_HEAD
-#define SBVR_HEAD 0
-#endif
-#ifndef SBVR_STREAM_AFTER_PREP
-#define SBVR_STREAM_AFTER_PREP 0
-#endif
-constexpr int kPrefetch = SBVR_PREFETCH;  // units requested ahead of the one being consumed
-constexpr int kTableRegs = 4;             // uint4 per thread while the coefficient table is staged
-constexpr size_t kMaxTableLds = kTableRegs * 16 * 256;   // largest coefficient table staged in LDS (16 KB)
 
 // Split-K accumulator: one 64-bit word per output, [count:8 | sum:56].  Every
 // workgroup adds (1 << 56) + (v + 2^47) with v = rint(partial * 2^30); integer
@@ -155,17 +142,15 @@ struct GemvArgs {
     const uint16_t *cache;
     const uint16_t *bias;
     uint16_t *out;
-    unsigned long long *acc;   // (M, N) split-K accumulators, all zero between calls
-    int M, N, K, G, L;
+    unsigned long long *acc;   // (M, N) split-K accumulators, all zero between calls (ksplit > 1 only)
+    int M, N, K, L;
     int gshift;           // a coefficient group is 128 << gshift elements
-    int n_tiles;          // workgroups along N
+    int idx16;            // line indices are uint16 (else uint8)
     int ksplit;           // workgroups along K
 #ifdef SBVR_TRACE
     unsigned long long *trace;   // 8 timestamps per workgroup (development builds only)
 #endif
 };
-
-__host__ __device__ constexpr size_t align16(size_t v) { return (v + 15) & ~static_cast<size_t>(15); }
 
 #ifdef SBVR_TRACE
 #define SBVR_STAMP(i)                                                         \
@@ -191,9 +176,6 @@ __device__ __forceinline__ int a_image_byte_offset(int k, int row)
     const int lane = 16 * ((kk >> 4) & 3) + row;
     return lane * 32 + p;
 }
-
-template <bool Wide> struct IdxType { typedef uint8_t type; };
-template <> struct IdxType<true> { typedef uint16_t type; };
 
 template <int S>
 struct Planes {
@@ -228,47 +210,13 @@ __device__ __forceinline__ Planes<S> load_planes(const uint32_t *p)
     return r;
 }
 
-// The S fp16 coefficients of one line, as floats.  P is an LDS or a global pointer.
-template <int S, typename P>
-__device__ __forceinline__ void load_coeffs(P cache, int line, float (&c)[S])
-{
-    P p = cache + static_cast<uint32_t>(line) * S;
-    if constexpr (S % 2 == 0) {
-        uint32_t v[S / 2];
-        if constexpr (S == 4) {
-            const uint2 t = *reinterpret_cast<const uint2 *>(p);
-            v[0] = t.x; v[1] = t.y;
-        } else if constexpr (S == 8) {
-            const uint4 t = *reinterpret_cast<const uint4 *>(p);
-            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-        } else {
-#pragma unroll
-            for (int j = 0; j < S / 2; ++j)
-                v[j] = reinterpret_cast<const uint32_t *>(p)[j];
-        }
-#pragma unroll
-        for (int j = 0; j < S / 2; ++j) {
-            c[2 * j] = h2f(static_cast<uint16_t>(v[j] & 0xffffu));
-            c[2 * j + 1] = h2f(static_cast<uint16_t>(v[j] >> 16));
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < S; ++j)
-            c[j] = h2f(p[j]);
-    }
-}
-
-// S planes, MT row tiles (4 batch rows each), a wave owns CT column tiles of 16
-// columns and the workgroup SP sub-groups of K; all CT*SP units of a wave are
-// loaded up front and consumed in order, so the code is straight-line and every
-// wait is for exactly the oldest load.
 // Waves per SIMD the register allocator is asked to leave room for: the queued
-// plane words (and line indices) of all units plus the working registers.
+// plane words, line indices and coefficients of all units, the activations, the
+// plane sums, the A operands and working registers.
 constexpr int gemv_waves(int S, int MT, int CT, int SP)
 {
-    // queued units, double-buffered products, A operands, sums, coefficients, scratch
-    const int live = CT * SP < kPrefetch + 1 ? CT * SP : kPrefetch + 1;
-    const int regs = live * (S + 1) + 8 * MT * S + 8 * MT + CT * MT + S + (S < 4 ? 28 : 12);
+    const int U = CT * SP;
+    const int regs = U * (S + 1 + (S + 1) / 2) + U * MT * S + 8 * SP * MT + 4 * SP * MT + 4 * MT * S + CT * MT + 32;
     const int w = 512 / regs;
     return w < 1 ? 1 : (w > 8 ? 8 : w);
 }
@@ -295,186 +243,169 @@ __device__ __forceinline__ long long to_fixed(float y)
     return (static_cast<long long>(static_cast<int>(hi)) << 24) + static_cast<long long>(static_cast<int>(lo));
 }
 
-// MODE 0: table in LDS, uint8 indices; 1: table in LDS, uint16 indices;
-//      2: table read from global memory (large tables), uint16 indices.
-// S planes, MT row tiles (4 batch rows each); a wave owns CT column tiles of 16
-// columns and the workgroup SP sub-groups of K.  All CT*SP units of a wave are
-// loaded up front and consumed in order: the code is straight-line, every wait
-// is for exactly the oldest load, and addresses are one base plus immediates.
-template <int S, int MT, int CT, int SP, int MODE>
-__global__ void __launch_bounds__(kThreads)
-__attribute__((amdgpu_waves_per_eu(gemv_waves(S, MT, CT, SP), gemv_waves(S, MT, CT, SP))))
+// S planes, MT row tiles (4 batch rows each), CT column tiles of 16 columns,
+// SP sub-groups (128 elements of K) per wave.  A workgroup owns 16*CT columns;
+// its waves (blockDim.x / 64 of them) split K: wave w of workgroup (nt, kp)
+// takes sub-groups [(kp * waves + w) * SP, +SP), i.e. U = CT*SP units of 1 KiB
+// of plane words.  The waves share nothing until their partial results meet in
+// LDS, so nothing in a wave waits for another wave before that.  Straight-line
+// code; every wait is for exactly the oldest outstanding load.  In a wave:
+//   1. all its requests at once: its activations (one dword per lane, row and
+//      sub-group), the line indices of its units, the plane words;
+//   2. the activations arrive first: they become the fp8 A operands (through
+//      a 2 KiB LDS buffer of the wave's own, which does the byte transpose);
+//   3. the indices arrive: the coefficient lines are gathered (vector loads
+//      queued behind the stream, they arrive right after the last plane words);
+//   4. every unit: four ANDs per plane word, MFMA, plane sums kept in registers;
+//   5. coefficients applied; partial results to LDS, barrier, summed in a fixed
+//      order by the first waves, written out (or added to the split-K words).
+template <int S, int MT, int CT, int SP>
+__global__ void __launch_bounds__(64 * kMaxWaves)
+__attribute__((amdgpu_waves_per_eu(gemv_waves(S, MT, CT, SP), 8)))
 sbvr_gemv_mfma_kernel(const GemvArgs a)
 {
-    constexpr bool TBL = MODE != 2;
-    typedef typename IdxType<MODE != 0>::type IdxT;
     extern __shared__ __align__(16) unsigned char smem[];
-    // smem: A images [SP][MT][64 lanes][32 bytes], scales [SP][MT*4] floats, then
-    // (TBL) a copy of the coefficient table
-    unsigned char *img = smem;
-    float *scales = reinterpret_cast<float *>(smem + SP * MT * 2048);
-    uint16_t *table = reinterpret_cast<uint16_t *>(smem + SP * MT * 2048 + align16(SP * MT * 16));
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int nt = blockIdx.x;   // workgroup along N
-    const int kp = blockIdx.y;   // workgroup along K
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int waves = static_cast<int>(blockDim.x >> 6);
     const int N = a.N, K = a.K;
     const int col = lane & 15;   // column inside a tile (B and D operands)
     const int blk = lane >> 4;   // word of the sub-group (B), batch row of the tile (D)
-    const int sg0 = kp * SP;     // first sub-group of this workgroup
-    // The wave owns columns [n_own, n_own + 16*CT).  It computes a full window
-    // of 16*CT columns; a window that would stick out of N is moved left, and
-    // the columns it then shares with its neighbour are left to the neighbour.
-    const int n_own = (nt * kWavesPerWG + wave) * CT * 16;
+    const int sg0 = (blockIdx.y * waves + wave) * SP;     // first sub-group of this wave
+    // The workgroup owns columns [n_own, n_own + 16*CT).  It computes a full
+    // window of 16*CT columns; a window that would stick out of N is moved left,
+    // and the columns it then shares with its neighbour are left to the neighbour.
+    const int n_own = blockIdx.x * CT * 16;
     const int n_base = min(n_own, N - CT * 16);
+    unsigned char *const mine = smem + wave * 2048;        // this wave's buffer
 
     SBVR_STAMP(0);
-    // -- 1. The vector-memory queue of a CU holds only a few tens of KB; a wave
-    //       that issues more stalls at the load until there is room.  So the
-    //       stream is started with the first kAhead units only, the small loads
-    //       every wave needs before its first MFMA (activations, table slice)
-    //       follow right behind them, and each later unit is requested kAhead
-    //       units before it is consumed.  Unit u = (sub-group u / CT, tile u % CT).
+    // -- 1. requests.  Unit u = (sub-group u / CT, column tile u % CT).
     constexpr int U = SP * CT;
-    constexpr int kAhead = U < kPrefetch ? U : kPrefetch;
-    Planes<S> q[U];
+    uint32_t xx[SP][MT][4];
+#pragma unroll
+    for (int sgi = 0; sgi < SP; ++sgi)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                xx[sgi][mt][r] = 0u;
+                if (mt * 4 + r < a.M)      // wave-uniform
+                    xx[sgi][mt][r] = reinterpret_cast<const uint32_t *>(
+                        a.x + static_cast<size_t>(mt * 4 + r) * K + static_cast<size_t>(sg0 + sgi) * kSub)[lane];
+            }
     int qline[U];
-    const uint32_t lane_w = (static_cast<uint32_t>(blk) * N + n_base + col) * S;   // words
-    const uint32_t lane_i = static_cast<uint32_t>(n_base + col);
-    auto request = [&](int u) {
-        const int sgi = u / CT, ct = u % CT;
-        const uint32_t *wrow = a.bvr + static_cast<size_t>(sg0 + sgi) * 4 * N * S;     // wave-uniform
-        const IdxT *irow = static_cast<const IdxT *>(a.idx) + static_cast<size_t>((sg0 + sgi) >> a.gshift) * N;
-        q[u] = load_planes<S>(wrow + lane_w + ct * 16 * S);
-#ifdef SBVR_HACK_NOIDX
-        qline[u] = (lane + u) & 255; (void)irow;
-#else
-        qline[u] = static_cast<int>(irow[lane_i + ct * 16]);
-#endif
-    };
-    constexpr int kHead = kAhead < SBVR_HEAD ? kAhead : SBVR_HEAD;   // units requested before the small loads
+    {
+        const uint32_t lane_i = static_cast<uint32_t>(n_base + col);
+        if (a.idx16) {
 #pragma unroll
-    for (int u = 0; u < kHead; ++u)
-        request(u);
-    constexpr int kTasks = SP * MT;          // image tasks per wave, at most (M <= 4*MT)
-    uint32_t xx[kTasks];
+            for (int u = 0; u < U; ++u)
+                qline[u] = static_cast<const uint16_t *>(a.idx)[static_cast<size_t>((sg0 + u / CT) >> a.gshift) * N + lane_i + (u % CT) * 16];
+        } else {
 #pragma unroll
-    for (int t = 0; t < kTasks; ++t) {
-        const int task = wave + kWavesPerWG * t;     // task = m * SP + sgi
-        const int m = task / SP, sgi = task % SP;
-#ifdef SBVR_HACK_NOPROLOGUE
-        xx[t] = lane * 77u + m; (void)sgi;
-#else
-        xx[t] = *reinterpret_cast<const uint32_t *>(
-            a.x + (m < a.M ? static_cast<size_t>(m) * K + static_cast<size_t>(sg0 + sgi) * kSub + 2 * lane : 0));
-#endif
-    }
-    uint4 treg[kTableRegs];
-    const int tvecs = a.L * S / 8;           // the table is a whole number of 16-byte vectors here
-    if constexpr (TBL) {
-#pragma unroll
-        for (int r = 0; r < kTableRegs; ++r) {
-            const int i = tid + r * kThreads;
-#ifdef SBVR_HACK_NOPROLOGUE
-            treg[r] = uint4{1u, 2u, 3u, 4u};
-#else
-            if (r * kThreads < tvecs)        // wave-uniform: small tables take one pass
-                treg[r] = reinterpret_cast<const uint4 *>(a.cache)[i < tvecs ? i : 0];
-#endif
+            for (int u = 0; u < U; ++u)
+                qline[u] = static_cast<const uint8_t *>(a.idx)[static_cast<size_t>((sg0 + u / CT) >> a.gshift) * N + lane_i + (u % CT) * 16];
         }
     }
-    for (int i = tid; i < SP * MT * 512; i += kThreads)
-        reinterpret_cast<uint32_t *>(img)[i] = 0u;
-    if constexpr (TBL) {
+    Planes<S> q[U];
+    {
+        const uint32_t lane_w = (static_cast<uint32_t>(blk) * N + n_base + col) * S;   // words
 #pragma unroll
-        for (int r = 0; r < kTableRegs; ++r) {
-            const int i = tid + r * kThreads;
-            if (i < tvecs)
-                reinterpret_cast<uint4 *>(table)[i] = treg[r];
+        for (int u = 0; u < U; ++u) {
+            const uint32_t *wrow = a.bvr + static_cast<size_t>(sg0 + u / CT) * 4 * N * S;     // wave-uniform
+            q[u] = load_planes<S>(wrow + lane_w + (u % CT) * 16 * S);
         }
     }
     SBVR_STAMP(1);
-    __syncthreads();
-    SBVR_STAMP(2);
 
-    // -- 2. A images of this workgroup's sub-groups: lane l turns elements 2l and
-    //       2l+1 of a (batch row, sub-group) into 3 fp8 terms each
+    // -- 2. A operands.  Lane l turns elements 2l and 2l+1 of a batch row into
+    //       3 fp8 terms each and drops the bytes where the MFMA wants them; the
+    //       lane then reads its 32 bytes back.  Row tiles go from the last one,
+    //       the only one that may have fewer than 4 rows, to the first, so a row
+    //       of the buffer that is not rewritten holds zeros.
+    v8i A[SP][MT];
+    float scale[SP][MT];         // of this lane's batch row (blk)
     {
-        // position of the lane's two elements in an image, and their B-nibble factors
         const int off0 = a_image_byte_offset(2 * lane, 0), off1 = a_image_byte_offset(2 * lane + 1, 0);
         const float fac0 = (lane & 1) ? 1.f : 4.f, fac1 = (lane & 1) ? 1.f : 2.f;
+        reinterpret_cast<uint4 *>(mine)[lane * 2] = uint4{0u, 0u, 0u, 0u};
+        reinterpret_cast<uint4 *>(mine)[lane * 2 + 1] = uint4{0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int t = 0; t < kTasks; ++t) {
-            const int task = wave + kWavesPerWG * t;
-            const int m = task / SP, sgi = task % SP;
-#ifdef SBVR_HACK_NOPREP
-            if (m < a.M && a.L < 0) {
-#else
-            if (m < a.M) {
-#endif
-                // 2^e puts the largest magnitude of the sub-group into [32, 64)
-                // (fp16 bits order like magnitudes; subnormals count as 2^-15)
-                const uint32_t amax = wave_umax(max(xx[t] & 0x7fffu, (xx[t] >> 16) & 0x7fffu));
-                const int eh = min(max(static_cast<int>(amax >> 10), 1), 30);
-                const int e = 20 - eh;
-                const float up = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
-                unsigned char *dst = img + (sgi * MT + (m >> 2)) * 2048 + (m & 3) * 4 * 32;
-                if (lane == 0)   // products come out as 2 * x * 2^e
-                    scales[sgi * (MT * 4) + m] = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
-                float z0 = h2f(static_cast<uint16_t>(xx[t] & 0xffffu)) * (up * fac0);
-                float z1 = h2f(static_cast<uint16_t>(xx[t] >> 16)) * (up * fac1);
-                // h1 + h2 + h3/256 == z exactly: each fp8 takes the next 4 significant
-                // bits, the last one of the residual scaled up out of the subnormals
+        for (int mt = MT - 1; mt >= 0; --mt)
 #pragma unroll
-                for (int term = 0; term < 3; ++term) {
-                    if (term == 2) {
-                        z0 *= kLastTermScale;
-                        z1 *= kLastTermScale;
+            for (int sgi = 0; sgi < SP; ++sgi) {
+                scale[sgi][mt] = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (mt * 4 + r < a.M) {      // wave-uniform
+                        const uint32_t v = xx[sgi][mt][r];
+                        // 2^e puts the largest magnitude of the sub-group into [32, 64)
+                        // (fp16 bits order like magnitudes; subnormals count as 2^-15)
+                        const uint32_t amax = wave_umax(max(v & 0x7fffu, (v >> 16) & 0x7fffu));
+                        const int eh = min(max(static_cast<int>(amax >> 10), 1), 30);
+                        const int e = 20 - eh;
+                        const float up = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
+                        if (blk == r)            // products come out as 2 * x * 2^e
+                            scale[sgi][mt] = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
+                        float z0 = h2f(static_cast<uint16_t>(v & 0xffffu)) * (up * fac0);
+                        float z1 = h2f(static_cast<uint16_t>(v >> 16)) * (up * fac1);
+                        // h1 + h2 + h3/256 == z exactly: each fp8 takes the next 4 significant
+                        // bits, the last one of the residual scaled up out of the subnormals
+#pragma unroll
+                        for (int term = 0; term < 3; ++term) {
+                            if (term == 2) {
+                                z0 *= kLastTermScale;
+                                z1 *= kLastTermScale;
+                            }
+                            const int b = __builtin_amdgcn_cvt_pk_fp8_f32(z0, z1, 0, false);
+                            z0 -= __builtin_amdgcn_cvt_f32_fp8(b, 0);
+                            z1 -= __builtin_amdgcn_cvt_f32_fp8(b, 1);
+                            mine[off0 + (r * 4 + term) * 32] = static_cast<unsigned char>(b & 0xff);
+                            mine[off1 + (r * 4 + term) * 32] = static_cast<unsigned char>((b >> 8) & 0xff);
+                        }
                     }
-                    const int b = __builtin_amdgcn_cvt_pk_fp8_f32(z0, z1, 0, false);
-                    z0 -= __builtin_amdgcn_cvt_f32_fp8(b, 0);
-                    z1 -= __builtin_amdgcn_cvt_f32_fp8(b, 1);
-                    dst[off0 + term * 32] = static_cast<unsigned char>(b & 0xff);
-                    dst[off1 + term * 32] = static_cast<unsigned char>((b >> 8) & 0xff);
                 }
+                A[sgi][mt] = *reinterpret_cast<const v8i *>(mine + lane * 32);
             }
+    }
+    SBVR_STAMP(2);
+
+    // -- 3. coefficient lines of the units (S fp16 each)
+    constexpr int CW = (S + 1) / 2;          // dwords per line
+    uint32_t cq[U][CW];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t line = static_cast<uint32_t>(min(qline[u], a.L - 1));
+        const uint16_t *p = a.cache + line * S;
+        if constexpr (S == 4) {
+            const uint2 t = *reinterpret_cast<const uint2 *>(p);
+            cq[u][0] = t.x; cq[u][1] = t.y;
+        } else if constexpr (S == 8) {
+            const uint4 t = *reinterpret_cast<const uint4 *>(p);
+            cq[u][0] = t.x; cq[u][1] = t.y; cq[u][2] = t.z; cq[u][3] = t.w;
+        } else if constexpr (S % 2 == 0) {
+#pragma unroll
+            for (int j = 0; j < CW; ++j)
+                cq[u][j] = reinterpret_cast<const uint32_t *>(p)[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < CW; ++j)
+                cq[u][j] = static_cast<uint32_t>(p[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(p[2 * j + 1]) << 16 : 0u);
         }
     }
-#if SBVR_STREAM_AFTER_PREP == 0
-#pragma unroll
-    for (int u = kHead; u < kAhead; ++u)
-        request(u);
-#endif
-    __syncthreads();
     SBVR_STAMP(3);
-#if SBVR_STREAM_AFTER_PREP == 1
-#pragma unroll
-    for (int u = kHead; u < kAhead; ++u)
-        request(u);
-#endif
 
-    // -- 3. consume the units: sub-group outer (A operand stays in registers),
-    //       column tile inner.  The MFMAs of a unit are issued before the
-    //       results of the previous unit are folded in, so their latency is covered.
-    float y[CT][MT];
+    // -- 4. the units: plane sums of every (unit, row tile, plane)
+    float ps[U][MT][S];
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            y[ct][mt] = 0.f;
-
-    v8i A[MT];
-    float sc[MT];
-    v4f D[2][MT][S];
-    float cprev[S];
-    float scprev[MT];
-    auto products = [&](int u, v4f (&Dn)[MT][S]) {
-        const Planes<S> &pl = q[u];
+    for (int u = 0; u < U; ++u) {
+        const int sgi = u / CT;
+        v4f D[MT][S];
 #pragma unroll
         for (int j = 0; j < S; ++j) {
-            const uint32_t w = pl.w[j];
+            const uint32_t w = q[u].w[j];
             v8i B;
             B[0] = static_cast<int>(w & 0x11111111u);
             B[1] = static_cast<int>(w & 0x22222222u);
@@ -484,124 +415,93 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 const v4f z = {0.f, 0.f, 0.f, 0.f};
-                Dn[mt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[mt], B, z, 0, 4, 0, 0, 0, 0);
+                D[mt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[sgi][mt], B, z, 0, 4, 0, 0, 0, 0);
             }
         }
-    };
-    auto coeffs_of = [&](int u, float (&c)[S]) {
-        const int line = min(qline[u], a.L - 1);
-        if constexpr (TBL)
-            load_coeffs<S>(static_cast<const uint16_t *>(table), line, c);
-        else
-            load_coeffs<S>(a.cache, line, c);
-    };
-    auto fold = [&](int ct, const v4f (&Dp)[MT][S]) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int j = 0; j < S; ++j) {
+                ps[u][mt][j] = fmaf(D[mt][j][2], 1.f / kLastTermScale, D[mt][j][0] + D[mt][j][1]);
+                asm volatile("" : "+v"(ps[u][mt][j]));       // keeps the units in program order
+            }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    SBVR_STAMP(4);
+
+    // -- 5. coefficients and scales; the lane holds column n_base + 16*ct + col
+    //       of batch row 4*mt + blk
+    float y[CT][MT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            y[ct][mt] = 0.f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int sgi = u / CT, ct = u % CT;
+        float c[S];
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+            c[j] = h2f(static_cast<uint16_t>(j & 1 ? cq[u][j / 2] >> 16 : cq[u][j / 2] & 0xffffu));
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             float acc = 0.f;
 #pragma unroll
             for (int j = 0; j < S; ++j)
-                acc = fmaf(cprev[j], fmaf(Dp[mt][j][2], 1.f / kLastTermScale, Dp[mt][j][0] + Dp[mt][j][1]), acc);
-            y[ct][mt] = fmaf(acc, scprev[mt], y[ct][mt]);
-            asm volatile("" : "+v"(y[ct][mt]));   // keeps the units in program order
+                acc = fmaf(c[j], ps[u][mt][j], acc);
+            y[ct][mt] = fmaf(acc, scale[sgi][mt], y[ct][mt]);
         }
-    };
-#pragma unroll
-    for (int u = 0; u < SP * CT; ++u) {
-        const int sgi = u / CT, ct = u % CT;
-        if (ct == 0) {
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                A[mt] = *reinterpret_cast<const v8i *>(img + (sgi * MT + mt) * 2048 + lane * 32);
-                sc[mt] = scales[sgi * (MT * 4) + mt * 4 + blk];
-            }
-        }
-        if (u + kAhead < U)
-            request(u + kAhead);
-        float c[S];
-        coeffs_of(u, c);
-        products(u, D[u & 1]);
-        if (u > 0)
-            fold((u - 1) % CT, D[(u - 1) & 1]);
-#pragma unroll
-        for (int j = 0; j < S; ++j)
-            cprev[j] = c[j];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            scprev[mt] = sc[mt];
-        __builtin_amdgcn_sched_barrier(0);
     }
-    fold((SP * CT - 1) % CT, D[(SP * CT - 1) & 1]);
-
-    SBVR_STAMP(4);
-#ifdef SBVR_HACK_NOFINAL
-    { float t = 0.f; for (int ct = 0; ct < CT; ++ct) for (int mt = 0; mt < MT; ++mt) t += y[ct][mt]; if (t == 123.456f) a.out[0] = 1; return; }
-#endif
-    // -- 4. results: direct when K is not split, else through the accumulators.
-    //       A lane holds column n_base + 16*ct + col of batch row 4*mt + blk.
-    const bool shifted = n_base != n_own;            // wave-uniform: window moved left at the edge of N
-    bool valid[CT][MT];
+    //       partial results meet in LDS: wave w's buffer holds [ct][mt][lane] floats
+    float *const red = reinterpret_cast<float *>(smem);
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-            valid[ct][mt] = (mt * 4 + blk < a.M) && (!shifted || n_base + ct * 16 + col >= n_own);
-    const size_t lane_o = static_cast<size_t>(blk) * N + n_base + col;
-    uint16_t *outp = a.out + lane_o;
-    auto store = [&](int ct, int mt, float v) {
-        uint16_t r = f2h(v);
-        if (a.bias)
-            r = hadd(r, a.bias[n_base + ct * 16 + col]);
-        outp[static_cast<size_t>(mt) * 4 * N + ct * 16] = r;
-    };
-    if (a.ksplit == 1) {
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-                if (valid[ct][mt])
-                    store(ct, mt, y[ct][mt]);
-        return;
-    }
-    unsigned long long *accp = a.acc + lane_o;
-    unsigned long long tot[CT][MT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            tot[ct][mt] = (1ull << 56) + static_cast<unsigned long long>(to_fixed(y[ct][mt]) + kAccBias);
-            unsigned long long old = 0ull;
-            if (valid[ct][mt])
-                old = __hip_atomic_fetch_add(accp + static_cast<size_t>(mt) * 4 * N + ct * 16, tot[ct][mt],
-                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            tot[ct][mt] += old;
-        }
-    }
+            red[wave * 512 + (ct * MT + mt) * 64 + lane] = y[ct][mt];
+    __syncthreads();
     SBVR_STAMP(5);
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            if (valid[ct][mt] && static_cast<int>(tot[ct][mt] >> 56) == a.ksplit) {
-                // the sum without the count and the ksplit biases, back to float:
-                // sum = hi * 2^24 + lo, both halves exact in fp32, one rounding
-                const long long sum = static_cast<long long>(tot[ct][mt] & ((1ull << 56) - 1)) -
-                                      (static_cast<long long>(a.ksplit) << 47);
-                const float hi = static_cast<float>(static_cast<int>(sum >> 24));
-                const float lo = static_cast<float>(static_cast<int>(sum & 0xffffff));
-                const float total = fmaf(hi, 1.f / (1 << (kAccFracBits - 24)), lo * (1.f / (1 << kAccFracBits)));
-                __hip_atomic_store(accp + static_cast<size_t>(mt) * 4 * N + ct * 16, 0ull,
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                store(ct, mt, total);
-            }
+
+    const bool shifted = n_base != n_own;            // window moved left at the edge of N
+    for (int o = wave; o < CT * MT; o += waves) {    // wave-uniform
+        const int ct = o / MT, mt = o % MT;
+        float total = 0.f;
+        for (int w = 0; w < waves; ++w)
+            total += red[w * 512 + o * 64 + lane];
+        const int n = n_base + ct * 16 + col, m = mt * 4 + blk;
+        const bool valid = m < a.M && (!shifted || n >= n_own);
+        const size_t at = static_cast<size_t>(m) * N + n;
+        if (a.ksplit > 1) {
+            // through the accumulators: the adder that completes the count converts
+            unsigned long long tot = (1ull << 56) + static_cast<unsigned long long>(to_fixed(total) + kAccBias);
+            unsigned long long old = 0ull;
+            if (valid)
+                old = __hip_atomic_fetch_add(a.acc + at, tot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            tot += old;
+            if (!valid || static_cast<int>(tot >> 56) != a.ksplit)
+                continue;
+            // the sum without the count and the ksplit biases, back to float:
+            // sum = hi * 2^24 + lo, both halves exact in fp32, one rounding
+            const long long sum = static_cast<long long>(tot & ((1ull << 56) - 1)) - (static_cast<long long>(a.ksplit) << 47);
+            const float hi = static_cast<float>(static_cast<int>(sum >> 24));
+            const float lo = static_cast<float>(static_cast<int>(sum & 0xffffff));
+            total = fmaf(hi, 1.f / (1 << (kAccFracBits - 24)), lo * (1.f / (1 << kAccFracBits)));
+            __hip_atomic_store(a.acc + at, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (!valid) {
+            continue;
         }
+        uint16_t r = f2h(total);
+        if (a.bias)
+            r = hadd(r, a.bias[n]);
+        a.out[at] = r;
     }
     SBVR_STAMP(6);
 }
 
 // Launch shape for the MFMA kernel.
 struct GemvPlan {
-    int CT, SP, n_tiles, ksplit, MT, mode;
+    int CT, SP, MT, waves, n_wgs, ksplit;
     size_t lds;
 };
 
@@ -612,59 +512,60 @@ int env_int(const char *name, int dflt)
 }
 
 // (CT, SP) pairs that have a kernel instance; see the dispatch below.
-constexpr int kShapes[][2] = {{1, 1}, {2, 1}, {4, 1}, {8, 1}, {2, 2}, {4, 2}, {8, 2}, {2, 4}, {4, 4}, {1, 8}, {2, 8}, {4, 8}, {8, 4}};
+constexpr int kShapes[][2] = {{1, 1}, {1, 2}, {1, 4}, {1, 7}, {2, 1}, {2, 2}, {2, 4}, {2, 7}, {4, 1}, {4, 2}, {4, 4}};
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
 
 bool shape_ok_for(int MT, int CT, int SP)
 {
     // larger batches keep to the smaller unit counts (register budget)
-    return MT == 1 || CT * SP <= 8;
+    // (and the partial results of a wave, CT*MT*64 floats, fit its 2 KiB buffer)
+    return CT * MT <= 8 && (MT == 1 || CT * SP * MT <= 16);
 }
 
-GemvPlan plan_gemv(int M, int N, int K, int S, int L, int idx_bytes, int cus)
+GemvPlan plan_gemv(int M, int N, int K, int S, int cus)
 {
     const int nsub = K / kSub;
     const int MT = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
     const int tiles16 = (N + 15) / 16;
     GemvPlan best{};
     double best_cost = 1e30;
-    const int eCT = env_int("SBVR_HIP_CT", 0), eSP = env_int("SBVR_HIP_SP", 0);
+    const int eCT = env_int("SBVR_HIP_CT", 0), eSP = env_int("SBVR_HIP_SP", 0), eW = env_int("SBVR_HIP_WAVES", 0);
     for (int i = 0; i < kNumShapes; ++i) {
         const int CT = kShapes[i][0], SP = kShapes[i][1];
-        if (nsub % SP || !shape_ok_for(MT, CT, SP) || nsub / SP > kMaxKsplit || CT * 16 > N)
+        if (nsub % SP || !shape_ok_for(MT, CT, SP) || CT * 16 > N)
             continue;
         if (eCT > 0 && eSP > 0 && (CT != eCT || SP != eSP))
             continue;
-        const int U = CT * SP;
-        const int n_tiles = (tiles16 + kWavesPerWG * CT - 1) / (kWavesPerWG * CT);
-        const int ksplit = nsub / SP;
-        const double wgs = static_cast<double>(n_tiles) * ksplit;
-        // A workgroup puts one wave on each SIMD, so `occ` workgroups fit a CU.
-        // Work that does not fit runs in a second round, which costs the whole
-        // start-up latency again: plans that fit in one round win.  Within a
-        // round every wave pays a fixed start-up (~4 units) and its share of
-        // the A images (~1.5 units per sub-group and batch row).
-        const int occ = gemv_waves(S, MT, CT, SP);
-        const double rounds = static_cast<double>((static_cast<long>(wgs) + static_cast<long>(cus) * occ - 1) /
-                                                  (static_cast<long>(cus) * occ));
-        const double per_wave = U + 4.0 + 1.5 * SP * M / kWavesPerWG;
-        const double waste = static_cast<double>(n_tiles) * kWavesPerWG * CT / tiles16;
-        const double fill = wgs < 1.5 * cus ? 1.5 * cus / wgs : 1.0;   // too few waves to cover latency
-        const double cost = rounds * (per_wave * waste / U * fill + 4.0 / U) + 0.01 * ksplit;
-        if (cost < best_cost) {
-            best_cost = cost;
-            best = GemvPlan{CT, SP, n_tiles, ksplit, MT, 0, 0};
+        const int parts = nsub / SP;             // wave-sized pieces of K
+        const int n_wgs = (tiles16 + CT - 1) / CT;
+        for (int waves = 1; waves <= kMaxWaves; ++waves) {
+            if (parts % waves || parts / waves > kMaxKsplit || (eW > 0 && waves != eW))
+                continue;
+            const int ksplit = parts / waves;
+            const int U = CT * SP;
+            const double total_waves = static_cast<double>(n_wgs) * parts;
+            // Per-wave cost in units of one streamed unit: the units, a fixed
+            // start-up, the A operands (one per sub-group and batch row).  A
+            // split along K through the accumulators costs every workgroup a
+            // round trip; too few waves leave load slots empty; work beyond one
+            // resident round (8 waves per SIMD) pays the start-up again.
+            const double per_wave = U + 3.0 + 0.7 * SP * M;
+            const double waste = static_cast<double>(n_wgs) * CT / tiles16;
+            const double resident = 32.0 * cus;
+            const double rounds = total_waves <= resident ? 1.0 : total_waves / resident + 0.5;
+            const double fill = total_waves < 8.0 * cus ? 8.0 * cus / total_waves : 1.0;
+            const double wg_balance = n_wgs * static_cast<double>(ksplit) < cus ? 1.3 : 1.0;
+            double cost = per_wave * waste / U * fill * rounds * wg_balance;
+            if (ksplit > 1)
+                cost *= 1.25;
+            cost += 0.002 * waves;
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = GemvPlan{CT, SP, MT, waves, n_wgs, ksplit, 0};
+            }
         }
     }
-    best.lds = static_cast<size_t>(best.SP) * MT * 2048 + align16(static_cast<size_t>(best.SP) * MT * 16);
-    const size_t table = static_cast<size_t>(L) * S * sizeof(uint16_t);
-    const bool in_lds = table <= kMaxTableLds && table % 16 == 0;
-    if (in_lds) {
-        best.lds += table;
-        best.mode = idx_bytes == 2 ? 1 : 0;
-    } else {
-        best.mode = idx_bytes == 2 ? 2 : -1;   // no kernel for a big table behind uint8 indices (cannot happen: L <= 256)
-    }
+    best.lds = static_cast<size_t>(best.waves) * 2048;
     return best;
 }
 
@@ -673,35 +574,27 @@ bool mfma_path_ok(int M, int N, int K, int S, int G)
     // 32-bit element offsets into bvr
     return M >= 1 && M <= kMaxM && N >= 16 && K % kSub == 0 && G % kSub == 0 && ((G / kSub) & (G / kSub - 1)) == 0 &&
            (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) &&
-           static_cast<double>(K / 32) * N * S < 2147483648.0 && K / kSub <= kMaxKsplit;
+           static_cast<double>(K / 32) * N * S < 2147483648.0;
 }
 
 template <int S, int MT, int CT, int SP>
 hipError_t launch_gemv_inst(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
-    const dim3 grid(static_cast<unsigned>(p.n_tiles), static_cast<unsigned>(p.ksplit)), block(kThreads);
-    if (p.mode == 0)
-        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, 0>), grid, block, p.lds, st, a);
-#ifndef SBVR_FAST_BUILD
-    else if (p.mode == 1)
-        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, 1>), grid, block, p.lds, st, a);
-    else
-        hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, 2>), grid, block, p.lds, st, a);
-#endif
+    const dim3 grid(static_cast<unsigned>(p.n_wgs), static_cast<unsigned>(p.ksplit)), block(64 * p.waves);
+    hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP>), grid, block, p.lds, st, a);
     return hipGetLastError();
 }
 
 template <int S, int MT>
 hipError_t launch_gemv_shape(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
-#define SBVR_SHAPE(ct, sp)                  \
-    if (p.CT == ct && p.SP == sp)           \
-        return launch_gemv_inst<S, MT, ct, sp>(a, p, st)
-    SBVR_SHAPE(1, 1); SBVR_SHAPE(2, 1); SBVR_SHAPE(4, 1); SBVR_SHAPE(8, 1);
-    SBVR_SHAPE(2, 2); SBVR_SHAPE(4, 2); SBVR_SHAPE(2, 4); SBVR_SHAPE(1, 8);
-    if constexpr (MT == 1) {
-        SBVR_SHAPE(8, 2); SBVR_SHAPE(4, 4); SBVR_SHAPE(2, 8); SBVR_SHAPE(4, 8); SBVR_SHAPE(8, 4);
-    }
+#define SBVR_SHAPE(ct, sp)                                  \
+    if constexpr (ct * MT <= 8 && (ct * sp * MT <= 16 || MT == 1)) \
+        if (p.CT == ct && p.SP == sp)                       \
+            return launch_gemv_inst<S, MT, ct, sp>(a, p, st)
+    SBVR_SHAPE(1, 1); SBVR_SHAPE(1, 2); SBVR_SHAPE(1, 4); SBVR_SHAPE(1, 7);
+    SBVR_SHAPE(2, 1); SBVR_SHAPE(2, 2); SBVR_SHAPE(2, 4); SBVR_SHAPE(2, 7);
+    SBVR_SHAPE(4, 1); SBVR_SHAPE(4, 2); SBVR_SHAPE(4, 4);
 #undef SBVR_SHAPE
     return hipErrorInvalidConfiguration;
 }
@@ -711,26 +604,27 @@ hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
     switch (p.MT) {
     case 1: return launch_gemv_shape<S, 1>(a, p, st);
+#ifndef SBVR_FAST_BUILD
     case 2: return launch_gemv_shape<S, 2>(a, p, st);
     default: return launch_gemv_shape<S, 4>(a, p, st);
+#else
+    default: return hipErrorInvalidConfiguration;
+#endif
     }
 }
 
 hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
-#ifdef SBVR_FAST_BUILD      // development builds: one instantiation family only
-    if (S == 4 && p.MT == 1 && p.mode == 0)
-        return launch_gemv_shape<4, 1>(a, p, st);
-    return hipErrorInvalidConfiguration;
-#else
     switch (S) {
+    case 4: return launch_gemv_mt<4>(a, p, st);
+#ifndef SBVR_FAST_BUILD      // development builds: one plane count only
     case 2: return launch_gemv_mt<2>(a, p, st);
     case 3: return launch_gemv_mt<3>(a, p, st);
-    case 4: return launch_gemv_mt<4>(a, p, st);
     case 6: return launch_gemv_mt<6>(a, p, st);
-    default: return launch_gemv_mt<8>(a, p, st);
-    }
+    case 8: return launch_gemv_mt<8>(a, p, st);
 #endif
+    default: return hipErrorInvalidConfiguration;
+    }
 }
 
 int current_cus()
@@ -876,8 +770,8 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
     const bool aligned = reinterpret_cast<uintptr_t>(bvr) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(coeff_cache) % 16 == 0;
     if (!(flags & 1) && aligned && mfma_path_ok(M, N, K, S, G)) {
-        const GemvPlan p = plan_gemv(M, N, K, S, L, idx_bytes, current_cus());
-        if (p.CT > 0 && p.mode >= 0) {
+        const GemvPlan p = plan_gemv(M, N, K, S, current_cus());
+        if (p.CT > 0) {
         GemvArgs a{};
         a.x = static_cast<const uint16_t *>(x);
         a.bvr = bvr;
@@ -885,9 +779,10 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
         a.cache = static_cast<const uint16_t *>(coeff_cache);
         a.bias = static_cast<const uint16_t *>(bias);
         a.out = static_cast<uint16_t *>(out);
-        a.M = M; a.N = N; a.K = K; a.G = G; a.L = L;
+        a.M = M; a.N = N; a.K = K; a.L = L;
         a.gshift = __builtin_ctz(static_cast<unsigned>(G / kSub));
-        a.n_tiles = p.n_tiles; a.ksplit = p.ksplit;
+        a.idx16 = idx_bytes == 2;
+        a.ksplit = p.ksplit;
 #ifdef SBVR_TRACE
         a.trace = g_trace;
 #endif
@@ -901,7 +796,7 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
         }
         const hipError_t e = launch_gemv(S, a, p, st);
         if (e != hipSuccess)
-            return fail(SBVR_HIP_ELAUNCH, "gemv launch (CT=%d SP=%d MT=%d): %s", p.CT, p.SP, p.MT, hipGetErrorString(e));
+            return fail(SBVR_HIP_ELAUNCH, "gemv launch (CT=%d SP=%d MT=%d waves=%d ksplit=%d): %s", p.CT, p.SP, p.MT, p.waves, p.ksplit, hipGetErrorString(e));
         return SBVR_HIP_OK;
         }
     }
