@@ -522,14 +522,27 @@ bool shape_ok_for(int MT, int CT, int SP)
     return CT * MT <= 8 && (MT == 1 || CT * SP * MT <= 16);
 }
 
+// Picks the launch shape.  Measured on MI355X (Llama-3-8B layer shapes, batch 1),
+// all sensible shapes are within a few percent of each other once these hold:
+//  - about 4 units per wave when there is enough work for 2048 such waves,
+//    fewer otherwise, with as many of them as possible along N (one sub-group
+//    per wave means one set of A operands per wave);
+//  - at least two workgroups per CU, so K is split across workgroups (through
+//    the accumulators) when N alone does not give that many;
+//  - the largest workgroup that keeps that, but no more than 8 waves when the
+//    waves do not all fit on the chip at once (finer placement).
 GemvPlan plan_gemv(int M, int N, int K, int S, int cus)
 {
     const int nsub = K / kSub;
     const int MT = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
     const int tiles16 = (N + 15) / 16;
+    const int eCT = env_int("SBVR_HIP_CT", 0), eSP = env_int("SBVR_HIP_SP", 0), eW = env_int("SBVR_HIP_WAVES", 0);
+    const long units = static_cast<long>(tiles16) * nsub;
+    int want = units >= 4L * 2048 ? 4 : (units >= 2L * 2048 ? 2 : 1);
+    while (want > 1 && !shape_ok_for(MT, want, 1))
+        want /= 2;
     GemvPlan best{};
     double best_cost = 1e30;
-    const int eCT = env_int("SBVR_HIP_CT", 0), eSP = env_int("SBVR_HIP_SP", 0), eW = env_int("SBVR_HIP_WAVES", 0);
     for (int i = 0; i < kNumShapes; ++i) {
         const int CT = kShapes[i][0], SP = kShapes[i][1];
         if (nsub % SP || !shape_ok_for(MT, CT, SP) || CT * 16 > N)
@@ -538,27 +551,24 @@ GemvPlan plan_gemv(int M, int N, int K, int S, int cus)
             continue;
         const int parts = nsub / SP;             // wave-sized pieces of K
         const int n_wgs = (tiles16 + CT - 1) / CT;
+        const long total_waves = static_cast<long>(n_wgs) * parts;
+        const int max_waves = total_waves > 32L * cus ? 8 : kMaxWaves;
         for (int waves = 1; waves <= kMaxWaves; ++waves) {
             if (parts % waves || parts / waves > kMaxKsplit || (eW > 0 && waves != eW))
                 continue;
             const int ksplit = parts / waves;
             const int U = CT * SP;
-            const double total_waves = static_cast<double>(n_wgs) * parts;
-            // Per-wave cost in units of one streamed unit: the units, a fixed
-            // start-up, the A operands (one per sub-group and batch row).  A
-            // split along K through the accumulators costs every workgroup a
-            // round trip; too few waves leave load slots empty; work beyond one
-            // resident round (8 waves per SIMD) pays the start-up again.
-            const double per_wave = U + 3.0 + 0.7 * SP * M;
-            const double waste = static_cast<double>(n_wgs) * CT / tiles16;
-            const double resident = 32.0 * cus;
-            const double rounds = total_waves <= resident ? 1.0 : total_waves / resident + 0.5;
-            const double fill = total_waves < 8.0 * cus ? 8.0 * cus / total_waves : 1.0;
-            const double wg_balance = n_wgs * static_cast<double>(ksplit) < cus ? 1.3 : 1.0;
-            double cost = per_wave * waste / U * fill * rounds * wg_balance;
-            if (ksplit > 1)
-                cost *= 1.25;
-            cost += 0.002 * waves;
+            double cost = 0.0;
+            cost += U == want ? 0.0 : (U < want ? 2.0 * (want - U) : 1.0 * (U - want));
+            cost += 0.5 * (SP - 1);                                          // A operands per wave
+            cost += static_cast<double>(n_wgs) * CT / tiles16 - 1.0;        // columns computed twice at the edge of N
+            if (static_cast<long>(n_wgs) * ksplit < 2L * cus)
+                cost += 3.0 * (1.0 - static_cast<double>(n_wgs) * ksplit / (2.0 * cus));
+            if (waves > max_waves)
+                cost += 1.0;
+            cost -= 0.01 * waves;                                            // larger workgroups, fewer accumulations
+            if (eCT > 0 && eSP > 0 && eW > 0)
+                cost = 0.0;
             if (cost < best_cost) {
                 best_cost = cost;
                 best = GemvPlan{CT, SP, MT, waves, n_wgs, ksplit, 0};
@@ -772,6 +782,8 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
     if (!(flags & 1) && aligned && mfma_path_ok(M, N, K, S, G)) {
         const GemvPlan p = plan_gemv(M, N, K, S, current_cus());
         if (p.CT > 0) {
+        if (env_int("SBVR_HIP_SHOW_PLAN", 0))
+            fprintf(stderr, "sbvr_hip plan M=%d N=%d K=%d S=%d: CT=%d SP=%d MT=%d waves=%d wgs=%d ksplit=%d\n", M, N, K, S, p.CT, p.SP, p.MT, p.waves, p.n_wgs, p.ksplit);
         GemvArgs a{};
         a.x = static_cast<const uint16_t *>(x);
         a.bvr = bvr;
