@@ -12,8 +12,11 @@ one weight copy; consecutive steps walk through COPIES distinct weight copies
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 prints one JSON line: whole-job throughput in GB/s of algorithmic bytes, the
-roofline of the kernel (HIP events on the launch stream) and the CPU baseline
-(the x86 port of the reference's timed CPU kernel, on the host's own cores).
+roofline of the kernel (HIP events on the launch stream), the second half of
+the metric ("decode": tokens/s of a random-init Llama-3-8B-shaped decoder whose
+linears are SBVR-encoded, 128-token prompt + 128 greedy tokens) and the CPU
+baseline (the x86 port of the reference's timed CPU kernel on the host's own
+cores: the gate GEMV, and the linears of one token for the decode figure).
 """
 import argparse
 import json
@@ -101,7 +104,70 @@ def gpu_leg(steps, warmup):
     return wall_ms, event_ms, launcher, torch.cuda.get_device_name(0)
 
 
-def cpu_leg(budget_s=12.0):
+def decode_leg(prompt_tokens=128, new_tokens=128):
+    """Random-init Llama-3-8B-shaped decoder with SBVR linears (sbvr/decoder.py):
+    a 128-token uniform-random prompt, then 128 greedy tokens at batch 1, one
+    HIP-graph replay per token; the figure covers the new tokens only."""
+    import torch
+    from sbvr.decoder import LlamaShape, SbvrLlamaDecoder
+
+    shape = LlamaShape()
+    dec = SbvrLlamaDecoder(shape, "cuda:0", num_sums=NUM_SUMS, bvr_len=GROUP, lines=LINES,
+                           max_seq=prompt_tokens + new_tokens)
+    dec.capture()
+    prompt = torch.randint(0, shape.vocab, (prompt_tokens,), generator=torch.Generator().manual_seed(0))
+    best = None
+    for _ in range(2):
+        tokens, seconds = dec.generate(prompt, new_tokens)
+        best = seconds if best is None else min(best, seconds)
+    per_token = dec.bytes_per_token()
+    out = {
+        "tokens_per_s": round(new_tokens / best, 1),
+        "ms_per_token": round(best / new_tokens * 1e3, 4),
+        "prompt_tokens": prompt_tokens,
+        "new_tokens": new_tokens,
+        "bytes_per_token": per_token,
+        "achieved_GBps": round(per_token * new_tokens / best / 1e9, 1),
+        "frac_of_hbm_peak": round(per_token * new_tokens / best / 1e9 / HBM_PEAK_GBS, 4),
+        "model": f"Llama-3-8B shape ({shape.layers} layers, d={shape.hidden}, {shape.heads}q/{shape.kv_heads}kv heads, "
+                 f"ffn {shape.ffn}, vocab {shape.vocab}), random init, SBVR S={NUM_SUMS} G={GROUP} on q|k|v, o, gate|up, "
+                 "down; fp16 embedding and head",
+        "first_tokens": [int(t) for t in tokens[:4]],
+    }
+    del dec
+    torch.cuda.empty_cache()
+    return out
+
+
+def cpu_decode_estimate(threads, per_shape_budget_s=1.5):
+    """Time of the linears of one token on the host: the reference CPU kernel (x86 port)
+    on each of the seven layer shapes, times 32 layers.  Excludes head, norms and attention."""
+    import numpy as np
+    from oracle import sbvr_oracle as O
+
+    rng = np.random.default_rng(11)
+    shapes = {"q/o": (4096, 4096, 2), "k/v": (1024, 4096, 2), "gate/up": (14336, 4096, 2), "down": (4096, 14336, 1)}
+    total = 0.0
+    detail = {}
+    for name, (n, k, count) in shapes.items():
+        l_bvr = O.np_planes_to_default(rng.integers(0, 256, size=(4, k // 8), dtype=np.uint8), 1)
+        l_idx = rng.integers(0, 16, size=(k // GROUP, 1)).astype(np.uint8)
+        l_cache = (rng.standard_normal((16, 4)) * 0.3).astype(np.float16)
+        r_bvr = O.np_planes_to_v1(rng.integers(0, 256, size=(NUM_SUMS, n * k // 8), dtype=np.uint8), n)
+        r_idx = rng.integers(0, LINES, size=(k // GROUP, n)).astype(np.uint8)
+        r_cache = (rng.standard_normal((LINES, NUM_SUMS)) * 0.02).astype(np.float16)
+        args = (l_bvr, l_idx, l_cache, r_bvr, r_idx, r_cache, GROUP)
+        probe = O.PORT.time_mm_T_v1(*args, warmup=2, iters=3)
+        iters = max(5, int(per_shape_budget_s / max(probe, 1e-6)))
+        t = O.PORT.time_mm_T_v1(*args, warmup=3, iters=iters)
+        detail[name] = round(t * 1e6, 1)
+        total += count * t
+    per_token = 32 * total
+    return {"tokens_per_s_linears_only": round(1.0 / per_token, 2), "ms_per_token_linears_only": round(per_token * 1e3, 2),
+            "us_per_gemv": detail, "cores": threads}
+
+
+def cpu_leg(budget_s=12.0, decode=True):
     """The reference's CPU algorithm (both operands encoded, popcount of AND,
     fp16 coefficient products) ported to x86, timed on this host for about
     `budget_s` seconds at the same shape."""
@@ -126,6 +192,7 @@ def cpu_leg(budget_s=12.0):
     probe = O.PORT.time_mm_T_v1(*args, warmup=2, iters=3)
     iters = max(10, int(budget_s / max(probe, 1e-6)))
     per_call = O.PORT.time_mm_T_v1(*args, warmup=10, iters=iters)
+    decode_cpu = cpu_decode_estimate(threads) if decode else None
     O.PORT.finalize_pool()
     nbytes = algorithmic_bytes(N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH)
     return {
@@ -137,6 +204,7 @@ def cpu_leg(budget_s=12.0):
         "isa": O.PORT.isa(),
         "sample": f"{iters} timed calls (10 warm-ups) of the full 4096->14336 GEMV, both operands SBVR-encoded "
                   f"(S_l=4, S_r=4, group 128), reference CPU algorithm ported to x86, N split over {threads} pinned threads",
+        "decode": decode_cpu,
     }
 
 
@@ -146,6 +214,8 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the 8B decode tokens/s leg")
+    ap.add_argument("--decode-only", action="store_true", help="run only the 8B decode leg and print its figures")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size kernel that "
                          "hardware byte counters are scaled by when profiling")
@@ -153,6 +223,9 @@ def main():
     if a.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the path is single-GPU in this build (run with --gpus 1)")
 
+    if a.decode_only:
+        print(json.dumps({"metric": "8B decode tokens/s", "decode": decode_leg()}))
+        return
     if a.calibrate_copy:
         import torch
         src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda:0")
@@ -196,8 +269,10 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES,
         },
     }
+    if not a.no_decode:
+        line["decode"] = decode_leg()
     if not a.no_cpu:
-        line["cpu_baseline"] = cpu_leg()
+        line["cpu_baseline"] = cpu_leg(decode=not a.no_decode)
     print(json.dumps(line))
 
 

@@ -48,6 +48,11 @@ def _load():
     lib.sbvr_hip_linear_f16.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp, sz, i, vp]
     lib.sbvr_hip_row_deq_mm_T.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp]
     lib.sbvr_hip_mm_T.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
+    fp = ctypes.POINTER(ctypes.c_float)
+    lib.sbvr_hip_dec_add_rmsnorm_f16.argtypes = [vp, vp, vp, vp, i, ctypes.c_float, vp]
+    lib.sbvr_hip_dec_attention_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
+    lib.sbvr_hip_dec_silu_mul_f16.argtypes = [vp, vp, i, vp]
+    lib.sbvr_hip_dec_argmax_advance_f16.argtypes = [vp, i, vp, vp, vp, i, vp]
     _lib = lib
     return lib
 
@@ -204,3 +209,58 @@ def _sbvr_mm_T(l_bvr, l_coeff_idx, l_coeff_cache, r_bvr, r_coeff_idx, r_coeff_ca
                                  _idx_bytes(r_coeff_idx, Lr, "r_coeff_idx"), r_coeff_cache.data_ptr(),
                                  _bias_ptr(bias, N, dev), out.data_ptr(), M, N, K, Sl, Sr, G, Ll, Lr, _stream()))
     return out
+
+
+# -- single-token helpers of the decoder (include/sbvr_hip_decoder.h) ------------
+
+def _dec_check(rc, what):
+    if rc != 0:
+        raise SbvrHipError(f"libsbvr_hip: {what} failed with {rc}")
+
+
+def dec_add_rmsnorm(x, delta, weight, h, eps):
+    """x (n,) fp16 updated in place with `delta` (or None); h <- weight * norm(x)."""
+    for t, name in ((x, "x"), (weight, "weight"), (h, "h")) + (((delta, "delta"),) if delta is not None else ()):
+        _want(t, name, torch.float16)
+    _dec_check(_load().sbvr_hip_dec_add_rmsnorm_f16(x.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                                     weight.data_ptr(), h.data_ptr(), x.numel(), float(eps),
+                                                     _stream()), "add_rmsnorm")
+    return h
+
+
+def dec_attention(qkv, cos, sin, pos, kcache, vcache, ctx, heads, kv_heads, head_dim):
+    """Rotary embedding, cache append at *pos and attention of the new token."""
+    for t, name in ((qkv, "qkv"), (kcache, "kcache"), (vcache, "vcache"), (ctx, "ctx")):
+        _want(t, name, torch.float16)
+    _want(cos, "cos", torch.float32)
+    _want(sin, "sin", torch.float32)
+    _want(pos, "pos", torch.int64)
+    max_seq = kcache.shape[1]
+    if kcache.shape != (kv_heads, max_seq, head_dim) or vcache.shape != kcache.shape or \
+            cos.shape != (max_seq, head_dim // 2) or sin.shape != cos.shape or \
+            qkv.numel() != (heads + 2 * kv_heads) * head_dim or ctx.numel() != heads * head_dim:
+        raise SbvrHipError("dec_attention: tensor shapes do not match heads/kv_heads/head_dim/max_seq")
+    _dec_check(_load().sbvr_hip_dec_attention_f16(qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), pos.data_ptr(),
+                                                   kcache.data_ptr(), vcache.data_ptr(), ctx.data_ptr(), heads,
+                                                   kv_heads, head_dim, max_seq, _stream()), "attention")
+    return ctx
+
+
+def dec_silu_mul(gate_up, out):
+    _want(gate_up, "gate_up", torch.float16)
+    _want(out, "out", torch.float16)
+    if gate_up.numel() != 2 * out.numel():
+        raise SbvrHipError("dec_silu_mul: gate_up must hold 2 * out.numel() elements")
+    _dec_check(_load().sbvr_hip_dec_silu_mul_f16(gate_up.data_ptr(), out.data_ptr(), out.numel(), _stream()),
+               "silu_mul")
+    return out
+
+
+def dec_argmax_advance(logits, token, generated, pos):
+    """token <- argmax(logits); generated[pos] <- token; pos <- pos + 1 (all on the device)."""
+    _want(logits, "logits", torch.float16)
+    for t, name in ((token, "token"), (generated, "generated"), (pos, "pos")):
+        _want(t, name, torch.int64)
+    _dec_check(_load().sbvr_hip_dec_argmax_advance_f16(logits.data_ptr(), logits.numel(), token.data_ptr(),
+                                                        generated.data_ptr(), pos.data_ptr(), generated.numel(),
+                                                        _stream()), "argmax_advance")

@@ -10,8 +10,8 @@ import torch
 
 
 def make_lines(num_lines, num_sums, sigma=0.02, seed=0):
-    """(num_lines, num_sums) fp16 table: c_j = b + s * r^j / spread, r in
-    (-2.1, -0.52), sorted by |c_j|."""
+    """(num_lines, num_sums) fp16 table: c_j = s * (r^j - mean_j r^j) / spread + b / num_sums,
+    r in (-2.1, -0.52), sorted by |c_j|."""
     rng = np.random.default_rng(seed)
     r = -rng.uniform(0.52, 2.09, size=(num_lines, 1))
     base = r ** np.arange(num_sums)[None, :]
@@ -20,7 +20,11 @@ def make_lines(num_lines, num_sums, sigma=0.02, seed=0):
     spread = sums.max(1, keepdims=True) - sums.min(1, keepdims=True)
     s = rng.uniform(4.0, 7.0, size=(num_lines, 1)) * sigma
     b = rng.uniform(-0.3, 0.3, size=(num_lines, 1)) * sigma
-    lines = b + s * base / spread
+    lines = s * base / spread
+    # the encoder fits zero-mean weights, so the 2^S points of a line straddle zero; with
+    # Bernoulli(1/2) planes that takes coefficients summing to (almost) nothing, or every
+    # row of the decoded matrix would share one large offset
+    lines = lines - lines.mean(1, keepdims=True) + b / num_sums
     order = np.argsort(np.abs(lines), axis=1)
     lines = np.take_along_axis(lines, order, axis=1)
     return torch.from_numpy(lines.astype(np.float16))

@@ -134,7 +134,8 @@ def test_ops_refuse_cpu_tensors():
 # ------------------------------------------------------------------ C ABI
 
 def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "sbvr_hip.h")).read()
+    text = "".join(open(os.path.join(ROOT, "include", name)).read()
+                   for name in sorted(os.listdir(os.path.join(ROOT, "include"))) if name.endswith(".h"))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(sbvr_hip_\w+)\s*\(", text)))
 
