@@ -637,6 +637,231 @@ hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t 
     }
 }
 
+// ------------------------------------------------------------- MFMA prefill
+
+// Prefill path (M > 16): a dense contraction.  A workgroup of 4 waves owns a
+// 256 x 128 tile of the output; per step of 64 along K it
+//   * copies the 256 x 64 activations to LDS as they are,
+//   * decodes the 128 x 64 weights to fp16 in LDS: thread (column, word) holds
+//     the S plane words of one 32-bit word of K and the coefficient line of its
+//     group, and forms w = sum_j (bit_j ? c_j : 0), two elements (k, k+16) per
+//     packed fp16 operation: (word >> k) & 0x00010001 times the 16-bit pattern
+//     of c_j is that pattern, or zero, in each half;
+//   * runs v_mfma_f32_32x32x16_f16 over the two tiles (each wave 128 x 64 of
+//     the output, 8 accumulator blocks).
+// The loads of the next step are issued before the MFMAs of the current one.
+// Rows of both LDS tiles are 128 bytes; 16-byte chunk c of row r is stored at
+// chunk c ^ (r & 7), which keeps the 16-byte operand reads of a quarter wave on
+// different banks.
+constexpr int kGemmBM = 256, kGemmBN = 128, kGemmBK = 64, kGemmThreads = 256;
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+struct GemmArgs {
+    const uint16_t *x;
+    const uint32_t *bvr;
+    const void *idx;
+    const uint16_t *cache;
+    const uint16_t *bias;
+    uint16_t *out;
+    int M, N, K, L;
+    int steps_per_group;   // G / 64
+    int idx16;
+};
+
+template <int S>
+__global__ void __launch_bounds__(kGemmThreads, 2)
+sbvr_gemm_mfma_kernel(const GemmArgs a)
+{
+    __shared__ __align__(16) unsigned char As[kGemmBM * kGemmBK * 2];
+    __shared__ __align__(16) unsigned char Bs[kGemmBN * kGemmBK * 2];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int N = a.N, K = a.K, M = a.M;
+    const int n0 = blockIdx.x * kGemmBN, m0 = blockIdx.y * kGemmBM;
+    const int steps = K / kGemmBK;
+
+    // decode role: column bn of the tile, word bw (0/1) of the step
+    const int bn = tid & (kGemmBN - 1), bw = tid >> 7;
+    const int n_ld = min(n0 + bn, N - 1);
+    // copy role: 8 chunks of 16 bytes, chunk q = tid + 256 i -> row q / 8, chunk q % 8
+    const uint16_t *xrow[8];
+    int a_dst[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int q = tid + kGemmThreads * i, row = q >> 3, c = q & 7;
+        xrow[i] = a.x + static_cast<size_t>(min(m0 + row, M - 1)) * K + c * 8;
+        a_dst[i] = row * 128 + ((c ^ (row & 7)) << 4);
+    }
+
+    uint4 areg[8];
+    uint32_t wreg[S];
+    uint32_t creg[(S + 1) / 2];
+    int line_next = 0;      // line index of the step after the one in wreg/creg
+
+    auto load_line = [&](int step) -> int {
+        const size_t at = static_cast<size_t>(step / a.steps_per_group) * N + n_ld;
+        const int v = a.idx16 ? static_cast<int>(static_cast<const uint16_t *>(a.idx)[at])
+                              : static_cast<int>(static_cast<const uint8_t *>(a.idx)[at]);
+        return min(v, a.L - 1);
+    };
+    auto load_step = [&](int step, int line) {
+        const int k0 = step * kGemmBK;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            areg[i] = *reinterpret_cast<const uint4 *>(xrow[i] + k0);
+        const uint32_t *wp = a.bvr + (static_cast<size_t>(k0 / 32 + bw) * N + n_ld) * S;
+        const Planes<S> pl = load_planes<S>(wp);
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+            wreg[j] = pl.w[j];
+        const uint16_t *cp = a.cache + static_cast<size_t>(line) * S;
+#pragma unroll
+        for (int j = 0; j < (S + 1) / 2; ++j) {
+            if (S % 2 == 0 || 2 * j + 1 < S)
+                creg[j] = static_cast<uint32_t>(cp[2 * j]) | (static_cast<uint32_t>(cp[2 * j + 1]) << 16);
+            else
+                creg[j] = cp[2 * j];
+        }
+    };
+
+    v16f acc[4][2];
+#pragma unroll
+    for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[bi][bj][r] = 0.f;
+
+    load_step(0, load_line(0));
+    if (steps > 1)
+        line_next = load_line(1);
+
+    const int wm = wave >> 1, wn = wave & 1;
+    for (int step = 0; step < steps; ++step) {
+        // ---- decode this thread's 32 weights
+        uint32_t cbits[S];
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+            cbits[j] = j & 1 ? creg[j / 2] >> 16 : creg[j / 2] & 0xffffu;
+        uint32_t pr[16];         // pr[k] = {w[k], w[k+16]}
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+#ifdef SBVR_GEMM_HACK_NODEQ
+            pr[k] = wreg[0] + k;
+#else
+            // (bits k and k+16 of the plane word, one per half) * (fp16 pattern) = the pattern or zero
+            v2h v = __builtin_bit_cast(v2h, __umul24((wreg[0] >> k) & 0x00010001u, cbits[0]));
+#pragma unroll
+            for (int j = 1; j < S; ++j)
+                v = v + __builtin_bit_cast(v2h, __umul24((wreg[j] >> k) & 0x00010001u, cbits[j]));
+            pr[k] = __builtin_bit_cast(uint32_t, v);
+#endif
+        }
+        uint4 lo0, lo1, hi0, hi1;      // k 0..7, 8..15, 16..23, 24..31
+        lo0.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x05040100u);  lo0.y = __builtin_amdgcn_perm(pr[3], pr[2], 0x05040100u);
+        lo0.z = __builtin_amdgcn_perm(pr[5], pr[4], 0x05040100u);  lo0.w = __builtin_amdgcn_perm(pr[7], pr[6], 0x05040100u);
+        lo1.x = __builtin_amdgcn_perm(pr[9], pr[8], 0x05040100u);  lo1.y = __builtin_amdgcn_perm(pr[11], pr[10], 0x05040100u);
+        lo1.z = __builtin_amdgcn_perm(pr[13], pr[12], 0x05040100u); lo1.w = __builtin_amdgcn_perm(pr[15], pr[14], 0x05040100u);
+        hi0.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x07060302u);  hi0.y = __builtin_amdgcn_perm(pr[3], pr[2], 0x07060302u);
+        hi0.z = __builtin_amdgcn_perm(pr[5], pr[4], 0x07060302u);  hi0.w = __builtin_amdgcn_perm(pr[7], pr[6], 0x07060302u);
+        hi1.x = __builtin_amdgcn_perm(pr[9], pr[8], 0x07060302u);  hi1.y = __builtin_amdgcn_perm(pr[11], pr[10], 0x07060302u);
+        hi1.z = __builtin_amdgcn_perm(pr[13], pr[12], 0x07060302u); hi1.w = __builtin_amdgcn_perm(pr[15], pr[14], 0x07060302u);
+        {
+            unsigned char *brow = Bs + bn * 128;
+            const int sw = bn & 7, cb = bw * 4;
+            *reinterpret_cast<uint4 *>(brow + (((cb + 0) ^ sw) << 4)) = lo0;
+            *reinterpret_cast<uint4 *>(brow + (((cb + 1) ^ sw) << 4)) = lo1;
+            *reinterpret_cast<uint4 *>(brow + (((cb + 2) ^ sw) << 4)) = hi0;
+            *reinterpret_cast<uint4 *>(brow + (((cb + 3) ^ sw) << 4)) = hi1;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            *reinterpret_cast<uint4 *>(As + a_dst[i]) = areg[i];
+        __syncthreads();
+
+        // ---- next step's loads fly during the MFMAs
+        if (step + 1 < steps) {
+            load_step(step + 1, line_next);
+            if (step + 2 < steps)
+                line_next = load_line(step + 2);
+        }
+
+#pragma unroll
+        for (int ks = 0; ks < kGemmBK / 16; ++ks) {
+            const int c = 2 * ks + (lane >> 5);
+            v8h af[4], bf[2];
+#pragma unroll
+            for (int bi = 0; bi < 4; ++bi) {
+                const int row = wm * 128 + bi * 32 + (lane & 31);
+                af[bi] = *reinterpret_cast<const v8h *>(As + row * 128 + ((c ^ (row & 7)) << 4));
+            }
+#pragma unroll
+            for (int bj = 0; bj < 2; ++bj) {
+                const int colr = wn * 64 + bj * 32 + (lane & 31);
+                bf[bj] = *reinterpret_cast<const v8h *>(Bs + colr * 128 + ((c ^ (colr & 7)) << 4));
+            }
+#pragma unroll
+            for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+                for (int bj = 0; bj < 2; ++bj)
+#ifdef SBVR_GEMM_HACK_NOMFMA
+                    acc[bi][bj][0] += static_cast<float>(af[bi][0] + bf[bj][1]);
+#else
+                    acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[bi], bf[bj], acc[bi][bj], 0, 0, 0);
+#endif
+        }
+        __syncthreads();
+    }
+
+    // ---- D[i][j] sits in lane j + 32*((i/4)%2), register (i%4) + 4*(i/8)
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj) {
+        const int n = n0 + wn * 64 + bj * 32 + (lane & 31);
+        if (n >= N)
+            continue;
+        const uint16_t bias = a.bias ? a.bias[n] : 0;
+#pragma unroll
+        for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * 128 + bi * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < M) {
+                    uint16_t v = f2h(acc[bi][bj][r]);
+                    if (a.bias)
+                        v = hadd(v, bias);
+                    a.out[static_cast<size_t>(m) * N + n] = v;
+                }
+            }
+    }
+}
+
+bool gemm_path_ok(int M, int N, int K, int S, int G)
+{
+    return M > kMaxM && K % kGemmBK == 0 && G % kGemmBK == 0 && (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) &&
+           static_cast<double>(K / 32) * N * S < 2147483648.0;
+}
+
+hipError_t launch_gemm(int S, const GemmArgs &a, hipStream_t st)
+{
+    const dim3 grid(static_cast<unsigned>((a.N + kGemmBN - 1) / kGemmBN), static_cast<unsigned>((a.M + kGemmBM - 1) / kGemmBM));
+    const dim3 block(kGemmThreads);
+    switch (S) {
+    case 4: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<4>, grid, block, 0, st, a); break;
+#ifndef SBVR_FAST_BUILD
+    case 2: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<2>, grid, block, 0, st, a); break;
+    case 3: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<3>, grid, block, 0, st, a); break;
+    case 6: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<6>, grid, block, 0, st, a); break;
+    case 8: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<8>, grid, block, 0, st, a); break;
+#endif
+    default: return hipErrorInvalidConfiguration;
+    }
+    return hipGetLastError();
+}
+
 int current_cus()
 {
     int dev = 0;
@@ -811,6 +1036,23 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
             return fail(SBVR_HIP_ELAUNCH, "gemv launch (CT=%d SP=%d MT=%d waves=%d ksplit=%d): %s", p.CT, p.SP, p.MT, p.waves, p.ksplit, hipGetErrorString(e));
         return SBVR_HIP_OK;
         }
+    }
+
+    if (!(flags & 1) && aligned && gemm_path_ok(M, N, K, S, G) && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        GemmArgs g{};
+        g.x = static_cast<const uint16_t *>(x);
+        g.bvr = bvr;
+        g.idx = coeff_idx;
+        g.cache = static_cast<const uint16_t *>(coeff_cache);
+        g.bias = static_cast<const uint16_t *>(bias);
+        g.out = static_cast<uint16_t *>(out);
+        g.M = M; g.N = N; g.K = K; g.L = L;
+        g.steps_per_group = G / kGemmBK;
+        g.idx16 = idx_bytes == 2;
+        const hipError_t e = launch_gemm(S, g, st);
+        if (e != hipSuccess)
+            return fail(SBVR_HIP_ELAUNCH, "gemm launch: %s", hipGetErrorString(e));
+        return SBVR_HIP_OK;
     }
 
     const size_t total = static_cast<size_t>(M) * N;

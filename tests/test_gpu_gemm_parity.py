@@ -1,0 +1,102 @@
+"""Prefill path (M > 16: weights decoded to fp16 tiles in LDS, fp16 MFMA)
+against the oracle.  The path rounds each decoded weight to fp16 (as the
+reference's decode() does, sbvr/core.py:927-949) and accumulates in fp32; the
+bar is the stated 1e-2 relative on fp16 outputs."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def check(y_gpu, yd, what):
+    """1e-2 relative; outputs below half the RMS output are judged against that half.
+    Every decoded weight is an fp16 sum of up to S fp16 coefficients here (the reference's
+    decode() rounds its weights to fp16 too), so an output's error scales with the RMS
+    output, about 2e-3 of it at most, and not with its own (possibly cancelling) value."""
+    y = y_gpu.float().cpu().numpy().astype(np.float64)
+    rms = float(np.sqrt(np.mean(yd ** 2))) + 1e-30
+    err = np.abs(y - yd)
+    rel = err / np.maximum(np.abs(yd), 0.5 * rms)
+    assert rel.max() <= 1e-2, f"{what}: relative error {rel.max():.3e} > 1e-2 (abs/rms {err.max() / rms:.3e})"
+
+
+def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False):
+    import sbvr
+    from sbvr import synth
+    dev = torch.device("cuda:0")
+    bvr, idx, cache = synth.random_encoding(N, K, S, G, L, seed=seed)
+    gen = torch.Generator().manual_seed(seed + 1)
+    x = torch.randn((M, K), generator=gen).to(torch.float16)
+    b = (torch.randn((N,), generator=gen) * 0.3).to(torch.float16) if bias else None
+    y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev),
+                              None if b is None else b.to(dev), bvr_len=G)
+    torch.cuda.synchronize()
+    _, yd = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), G)
+    if b is not None:
+        yd = yd + b.numpy().astype(np.float64)
+    check(y, yd, f"N={N} K={K} S={S} G={G} M={M} L={L}")
+
+
+@pytest.mark.parametrize("M", [17, 64, 256, 300])
+def test_rows(oracle, M):
+    run_case(oracle, 256, 512, 4, 128, M, 256, seed=M)
+
+
+@pytest.mark.parametrize("S", [2, 3, 4, 6, 8])
+def test_planes(oracle, S):
+    run_case(oracle, 128, 512, S, 128, 96, 200, seed=10 + S)
+
+
+@pytest.mark.parametrize("G", [64, 128, 256, 512])
+def test_groups(oracle, G):
+    run_case(oracle, 256, 1024, 4, G, 40, 256, seed=20 + G)
+
+
+@pytest.mark.parametrize("N", [16, 100, 130, 1000])
+def test_ragged_n(oracle, N):
+    run_case(oracle, N, 256, 4, 128, 33, 64, seed=30 + N)
+
+
+def test_u16_index_and_bias(oracle):
+    run_case(oracle, 320, 768, 4, 128, 50, 3000, seed=41)
+    run_case(oracle, 320, 768, 3, 128, 50, 256, seed=42, bias=True)
+
+
+def test_two_tiles_each_way(oracle):
+    run_case(oracle, 384, 1024, 4, 128, 520, 256, seed=43)
+
+
+def test_matches_decode_path_rows():
+    """The same rows through the decode path (16 at a time) and the prefill path."""
+    import sbvr
+    from sbvr import synth
+    dev = torch.device("cuda:0")
+    N, K, M = 1024, 2048, 64
+    bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(N, K, 4, 128, 256, seed=50))
+    x = torch.randn((M, K), generator=torch.Generator().manual_seed(51)).to(torch.float16).to(dev)
+    big = sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, bvr_len=128).float()
+    small = torch.cat([sbvr._sbvr_linear_f16(x[i:i + 16].contiguous(), bvr, idx, cache, None, bvr_len=128)
+                       for i in range(0, M, 16)]).float()
+    rms = small.pow(2).mean().sqrt()
+    assert ((big - small).abs() / torch.maximum(small.abs(), rms)).max().item() < 4e-3
+
+
+def test_linearity_70b_width():
+    """At the 8192 -> 28672 shape the oracle is out of reach: f(x1 + x2) = f(x1) + f(x2)
+    for activations whose sum is exact in fp16, and row m of a large batch equals the
+    same row computed alone through the decode path."""
+    import sbvr
+    from sbvr import synth
+    dev = torch.device("cuda:0")
+    N, K, M = 28672, 8192, 256
+    bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(N, K, 4, 128, 256, seed=60))
+    g = torch.Generator().manual_seed(61)
+    x1 = (torch.randint(-64, 64, (M, K), generator=g).float() / 32).to(torch.float16).to(dev)
+    x2 = (torch.randint(-64, 64, (M, K), generator=g).float() / 32).to(torch.float16).to(dev)
+    f = lambda x: sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, bvr_len=128).float()
+    y1, y2, y12 = f(x1), f(x2), f((x1 + x2))
+    rms = y12.pow(2).mean().sqrt()
+    assert ((y12 - (y1 + y2)).abs() / torch.maximum(y12.abs(), rms)).max().item() < 4e-3
+    row = sbvr._sbvr_linear_f16(x1[7:8].contiguous(), bvr, idx, cache, None, bvr_len=128).float()
+    assert ((y1[7:8] - row).abs() / torch.maximum(row.abs(), rms)).max().item() < 4e-3
