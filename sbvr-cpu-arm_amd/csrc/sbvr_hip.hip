@@ -639,25 +639,30 @@ hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t 
 
 // ------------------------------------------------------------- MFMA prefill
 
-// Prefill path (M > 16): a dense contraction.  A workgroup of 4 waves owns a
-// 256 x 128 tile of the output; per step of 64 along K it
-//   * copies the 256 x 64 activations to LDS as they are,
-//   * decodes the 128 x 64 weights to fp16 in LDS: thread (column, word) holds
-//     the S plane words of one 32-bit word of K and the coefficient line of its
-//     group, and forms w = sum_j (bit_j ? c_j : 0), two elements (k, k+16) per
-//     packed fp16 operation: (word >> k) & 0x00010001 times the 16-bit pattern
-//     of c_j is that pattern, or zero, in each half;
-//   * runs v_mfma_f32_32x32x16_f16 over the two tiles (each wave 128 x 64 of
-//     the output, 8 accumulator blocks).
-// The loads of the next step are issued before the MFMAs of the current one.
-// Rows of both LDS tiles are 128 bytes; 16-byte chunk c of row r is stored at
-// chunk c ^ (r & 7), which keeps the 16-byte operand reads of a quarter wave on
+// Prefill path (M > 16): a dense contraction.  A workgroup owns a 256 x 128
+// tile of the output and walks K in steps of 64.  Its 8 waves have two jobs:
+//   * waves 4-7 produce the LDS tiles of step t+1 while step t is consumed:
+//     they copy the 256 x 64 activations as they are and decode the 128 x 64
+//     weights to fp16: thread (column, word) holds the S plane words of one
+//     32-bit word of K and the coefficient line of its group, and forms
+//     w = sum_j (bit_j ? c_j : 0), two elements (k, k+16) per packed fp16
+//     operation: (word >> k) & 0x00010001 times the 16-bit pattern of c_j is
+//     that pattern, or zero, in each half.  Their global loads run three steps
+//     ahead of the consumers, in three register sets used in rotation;
+//   * waves 0-3 run v_mfma_f32_32x32x16_f16 over the two tiles (each wave
+//     128 x 64 of the output, 8 accumulator blocks).
+// A SIMD holds one wave of each kind, so the decode (VALU) and the MFMAs
+// overlap.  Both tiles are double-buffered; one barrier per step.  Rows of the
+// LDS tiles are 128 bytes; 16-byte chunk c of row r is stored at chunk
+// c ^ (r & 7), which keeps the 16-byte operand reads of a quarter wave on
 // different banks.
-constexpr int kGemmBM = 256, kGemmBN = 128, kGemmBK = 64, kGemmThreads = 256;
+constexpr int kGemmBM = 256, kGemmBN = 128, kGemmBK = 64, kGemmThreads = 512;
+constexpr int kGemmATile = kGemmBM * kGemmBK * 2, kGemmBTile = kGemmBN * kGemmBK * 2;
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
 struct GemmArgs {
     const uint16_t *x;
@@ -672,61 +677,144 @@ struct GemmArgs {
 };
 
 template <int S>
-__global__ void __launch_bounds__(kGemmThreads, 2)
+__global__ void __launch_bounds__(kGemmThreads)
+__attribute__((amdgpu_waves_per_eu(2, 2)))
 sbvr_gemm_mfma_kernel(const GemmArgs a)
 {
-    __shared__ __align__(16) unsigned char As[kGemmBM * kGemmBK * 2];
-    __shared__ __align__(16) unsigned char Bs[kGemmBN * kGemmBK * 2];
+    extern __shared__ __align__(16) unsigned char gsm[];
+    unsigned char *const As = gsm;                       // 2 tiles
+    unsigned char *const Bs = gsm + 2 * kGemmATile;      // 2 tiles
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int N = a.N, K = a.K, M = a.M;
     const int n0 = blockIdx.x * kGemmBN, m0 = blockIdx.y * kGemmBM;
     const int steps = K / kGemmBK;
+    const int rounds = (steps + 2) / 3;                  // both kinds of waves run 3 * rounds steps (same barriers)
 
-    // decode role: column bn of the tile, word bw (0/1) of the step
-    const int bn = tid & (kGemmBN - 1), bw = tid >> 7;
-    const int n_ld = min(n0 + bn, N - 1);
-    // copy role: 8 chunks of 16 bytes, chunk q = tid + 256 i -> row q / 8, chunk q % 8
-    const uint16_t *xrow[8];
-    int a_dst[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int q = tid + kGemmThreads * i, row = q >> 3, c = q & 7;
-        xrow[i] = a.x + static_cast<size_t>(min(m0 + row, M - 1)) * K + c * 8;
-        a_dst[i] = row * 128 + ((c ^ (row & 7)) << 4);
-    }
-
-    uint4 areg[8];
-    uint32_t wreg[S];
-    uint32_t creg[(S + 1) / 2];
-    int line_next = 0;      // line index of the step after the one in wreg/creg
-
-    auto load_line = [&](int step) -> int {
-        const size_t at = static_cast<size_t>(step / a.steps_per_group) * N + n_ld;
-        const int v = a.idx16 ? static_cast<int>(static_cast<const uint16_t *>(a.idx)[at])
-                              : static_cast<int>(static_cast<const uint8_t *>(a.idx)[at]);
-        return min(v, a.L - 1);
-    };
-    auto load_step = [&](int step, int line) {
-        const int k0 = step * kGemmBK;
+    if (wave >= 4) {
+        // ------------------------------------------------------------ producers
+        const int pt = tid - 256;
+        const int bn = pt & (kGemmBN - 1), bw = pt >> 7;  // decode role: column of the tile, word of the step
+        const int n_ld = min(n0 + bn, N - 1);
+        // copy role: chunk q = pt + 256 i of the step's 2048 16-byte chunks: row q / 8, chunk q % 8
+        uint32_t xoff[8];
+        const int row0 = pt >> 3, c0 = pt & 7;
 #pragma unroll
         for (int i = 0; i < 8; ++i)
-            areg[i] = *reinterpret_cast<const uint4 *>(xrow[i] + k0);
-        const uint32_t *wp = a.bvr + (static_cast<size_t>(k0 / 32 + bw) * N + n_ld) * S;
-        const Planes<S> pl = load_planes<S>(wp);
-#pragma unroll
-        for (int j = 0; j < S; ++j)
-            wreg[j] = pl.w[j];
-        const uint16_t *cp = a.cache + static_cast<size_t>(line) * S;
-#pragma unroll
-        for (int j = 0; j < (S + 1) / 2; ++j) {
-            if (S % 2 == 0 || 2 * j + 1 < S)
-                creg[j] = static_cast<uint32_t>(cp[2 * j]) | (static_cast<uint32_t>(cp[2 * j + 1]) << 16);
-            else
-                creg[j] = cp[2 * j];
-        }
-    };
+            xoff[i] = static_cast<uint32_t>(min(m0 + row0 + 32 * i, M - 1)) * K + c0 * 8;     // M * K < 2^31 (checked)
+        const int a_dst = row0 * 128 + ((c0 ^ (row0 & 7)) << 4);       // + 4096 i
+        const int b_dst = bn * 128;
+        const int sw = bn & 7, cb = bw * 4;
 
+        constexpr int CW = (S + 1) / 2;
+        v4u areg0[8], areg1[8], areg2[8];                // three register sets, used in rotation
+        uint32_t wreg0[S], wreg1[S], wreg2[S];
+        uint32_t creg0[CW], creg1[CW], creg2[CW];
+        int line[2] = {0, 0};       // line index of the tile to be requested next, and of the one after
+
+        auto load_line = [&](int t) __attribute__((always_inline)) -> int {
+            const size_t at = static_cast<size_t>(t / a.steps_per_group) * N + n_ld;
+            const int v = a.idx16 ? static_cast<int>(static_cast<const uint16_t *>(a.idx)[at])
+                                  : static_cast<int>(static_cast<const uint8_t *>(a.idx)[at]);
+            return min(v, a.L - 1);
+        };
+        // global loads of tile t into one register set
+        auto request = [&](int t, v4u (&ar)[8], uint32_t (&wr)[S], uint32_t (&cr)[CW]) __attribute__((always_inline)) {
+            const int k0 = t * kGemmBK;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                ar[i] = *reinterpret_cast<const v4u *>(a.x + xoff[i] + k0);
+            const uint32_t *wp = a.bvr + (static_cast<size_t>(k0 / 32 + bw) * N + n_ld) * S;
+            const Planes<S> pl = load_planes<S>(wp);
+#pragma unroll
+            for (int j = 0; j < S; ++j)
+                wr[j] = pl.w[j];
+            const uint16_t *cp = a.cache + static_cast<size_t>(line[0]) * S;
+#pragma unroll
+            for (int j = 0; j < (S + 1) / 2; ++j) {
+                if (S % 2 == 0 || 2 * j + 1 < S)
+                    cr[j] = static_cast<uint32_t>(cp[2 * j]) | (static_cast<uint32_t>(cp[2 * j + 1]) << 16);
+                else
+                    cr[j] = cp[2 * j];
+            }
+            line[0] = line[1];
+            if (t + 2 < steps)
+                line[1] = load_line(t + 2);
+        };
+        // one register set -> LDS buffers t % 2
+        auto produce = [&](int t, const v4u (&ar)[8], const uint32_t (&wr)[S], const uint32_t (&cr)[CW]) __attribute__((always_inline)) {
+            unsigned char *At = As + (t & 1) * kGemmATile, *Bt = Bs + (t & 1) * kGemmBTile;
+            uint32_t cbits[S];
+#pragma unroll
+            for (int j = 0; j < S; ++j)
+                cbits[j] = j & 1 ? cr[j / 2] >> 16 : cr[j / 2] & 0xffffu;
+            uint32_t pr[16];         // pr[k] = {w[k], w[k+16]}
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                v2h v = __builtin_bit_cast(v2h, __umul24((wr[0] >> k) & 0x00010001u, cbits[0]));
+#pragma unroll
+                for (int j = 1; j < S; ++j)
+                    v = v + __builtin_bit_cast(v2h, __umul24((wr[j] >> k) & 0x00010001u, cbits[j]));
+                pr[k] = __builtin_bit_cast(uint32_t, v);
+            }
+            v4u q[4];                // k 0..7, 8..15 (low halves), 16..23, 24..31 (high halves)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t sel = h ? 0x07060302u : 0x05040100u;
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    q[2 * h + g].x = __builtin_amdgcn_perm(pr[8 * g + 1], pr[8 * g + 0], sel);
+                    q[2 * h + g].y = __builtin_amdgcn_perm(pr[8 * g + 3], pr[8 * g + 2], sel);
+                    q[2 * h + g].z = __builtin_amdgcn_perm(pr[8 * g + 5], pr[8 * g + 4], sel);
+                    q[2 * h + g].w = __builtin_amdgcn_perm(pr[8 * g + 7], pr[8 * g + 6], sel);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                *reinterpret_cast<v4u *>(Bt + b_dst + (((cb + c) ^ sw) << 4)) = q[c];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                *reinterpret_cast<v4u *>(At + a_dst + 4096 * i) = ar[i];
+        };
+#define SBVR_SET(n) areg##n, wreg##n, creg##n
+        line[0] = load_line(0);
+        if (steps > 1)
+            line[1] = load_line(1);
+        request(0, SBVR_SET(0));
+        if (steps > 1)
+            request(1, SBVR_SET(1));
+        if (steps > 2)
+            request(2, SBVR_SET(2));
+        produce(0, SBVR_SET(0));
+        __syncthreads();
+        // step i: the consumers read tile i; tile i+1 goes to the other buffers, tile i+3 is requested
+        for (int r = 0; r < rounds; ++r) {
+            const int i = 3 * r;
+            if (i + 1 < steps) {
+                if (i + 3 < steps)
+                    request(i + 3, SBVR_SET(0));
+                produce(i + 1, SBVR_SET(1));
+            }
+            __syncthreads();
+            if (i + 2 < steps) {
+                if (i + 4 < steps)
+                    request(i + 4, SBVR_SET(1));
+                produce(i + 2, SBVR_SET(2));
+            }
+            __syncthreads();
+            if (i + 3 < steps) {
+                if (i + 5 < steps)
+                    request(i + 5, SBVR_SET(2));
+                produce(i + 3, SBVR_SET(0));
+            }
+            __syncthreads();
+        }
+#undef SBVR_SET
+        return;
+    }
+
+    // ---------------------------------------------------------------- consumers
     v16f acc[4][2];
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi)
@@ -735,84 +823,29 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 acc[bi][bj][r] = 0.f;
-
-    load_step(0, load_line(0));
-    if (steps > 1)
-        line_next = load_line(1);
-
     const int wm = wave >> 1, wn = wave & 1;
-    for (int step = 0; step < steps; ++step) {
-        // ---- decode this thread's 32 weights
-        uint32_t cbits[S];
+    const int arow = wm * 128 + (lane & 31), brow = wn * 64 + (lane & 31);      // + 32 bi / bj: same row & 7
+    const int rsw = lane & 7, chi = lane >> 5;
+    __syncthreads();
+    for (int i = 0; i < 3 * rounds; ++i) {
+        if (i < steps) {
+            const unsigned char *At = As + (i & 1) * kGemmATile, *Bt = Bs + (i & 1) * kGemmBTile;
 #pragma unroll
-        for (int j = 0; j < S; ++j)
-            cbits[j] = j & 1 ? creg[j / 2] >> 16 : creg[j / 2] & 0xffffu;
-        uint32_t pr[16];         // pr[k] = {w[k], w[k+16]}
+            for (int ks = 0; ks < kGemmBK / 16; ++ks) {
+                const int coff = ((2 * ks + chi) ^ rsw) << 4;
+                v8h af[4], bf[2];
 #pragma unroll
-        for (int k = 0; k < 16; ++k) {
-#ifdef SBVR_GEMM_HACK_NODEQ
-            pr[k] = wreg[0] + k;
-#else
-            // (bits k and k+16 of the plane word, one per half) * (fp16 pattern) = the pattern or zero
-            v2h v = __builtin_bit_cast(v2h, __umul24((wreg[0] >> k) & 0x00010001u, cbits[0]));
-#pragma unroll
-            for (int j = 1; j < S; ++j)
-                v = v + __builtin_bit_cast(v2h, __umul24((wreg[j] >> k) & 0x00010001u, cbits[j]));
-            pr[k] = __builtin_bit_cast(uint32_t, v);
-#endif
-        }
-        uint4 lo0, lo1, hi0, hi1;      // k 0..7, 8..15, 16..23, 24..31
-        lo0.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x05040100u);  lo0.y = __builtin_amdgcn_perm(pr[3], pr[2], 0x05040100u);
-        lo0.z = __builtin_amdgcn_perm(pr[5], pr[4], 0x05040100u);  lo0.w = __builtin_amdgcn_perm(pr[7], pr[6], 0x05040100u);
-        lo1.x = __builtin_amdgcn_perm(pr[9], pr[8], 0x05040100u);  lo1.y = __builtin_amdgcn_perm(pr[11], pr[10], 0x05040100u);
-        lo1.z = __builtin_amdgcn_perm(pr[13], pr[12], 0x05040100u); lo1.w = __builtin_amdgcn_perm(pr[15], pr[14], 0x05040100u);
-        hi0.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x07060302u);  hi0.y = __builtin_amdgcn_perm(pr[3], pr[2], 0x07060302u);
-        hi0.z = __builtin_amdgcn_perm(pr[5], pr[4], 0x07060302u);  hi0.w = __builtin_amdgcn_perm(pr[7], pr[6], 0x07060302u);
-        hi1.x = __builtin_amdgcn_perm(pr[9], pr[8], 0x07060302u);  hi1.y = __builtin_amdgcn_perm(pr[11], pr[10], 0x07060302u);
-        hi1.z = __builtin_amdgcn_perm(pr[13], pr[12], 0x07060302u); hi1.w = __builtin_amdgcn_perm(pr[15], pr[14], 0x07060302u);
-        {
-            unsigned char *brow = Bs + bn * 128;
-            const int sw = bn & 7, cb = bw * 4;
-            *reinterpret_cast<uint4 *>(brow + (((cb + 0) ^ sw) << 4)) = lo0;
-            *reinterpret_cast<uint4 *>(brow + (((cb + 1) ^ sw) << 4)) = lo1;
-            *reinterpret_cast<uint4 *>(brow + (((cb + 2) ^ sw) << 4)) = hi0;
-            *reinterpret_cast<uint4 *>(brow + (((cb + 3) ^ sw) << 4)) = hi1;
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            *reinterpret_cast<uint4 *>(As + a_dst[i]) = areg[i];
-        __syncthreads();
-
-        // ---- next step's loads fly during the MFMAs
-        if (step + 1 < steps) {
-            load_step(step + 1, line_next);
-            if (step + 2 < steps)
-                line_next = load_line(step + 2);
-        }
-
-#pragma unroll
-        for (int ks = 0; ks < kGemmBK / 16; ++ks) {
-            const int c = 2 * ks + (lane >> 5);
-            v8h af[4], bf[2];
-#pragma unroll
-            for (int bi = 0; bi < 4; ++bi) {
-                const int row = wm * 128 + bi * 32 + (lane & 31);
-                af[bi] = *reinterpret_cast<const v8h *>(As + row * 128 + ((c ^ (row & 7)) << 4));
-            }
-#pragma unroll
-            for (int bj = 0; bj < 2; ++bj) {
-                const int colr = wn * 64 + bj * 32 + (lane & 31);
-                bf[bj] = *reinterpret_cast<const v8h *>(Bs + colr * 128 + ((c ^ (colr & 7)) << 4));
-            }
-#pragma unroll
-            for (int bi = 0; bi < 4; ++bi)
+                for (int bi = 0; bi < 4; ++bi)
+                    af[bi] = *reinterpret_cast<const v8h *>(At + (arow + 32 * bi) * 128 + coff);
 #pragma unroll
                 for (int bj = 0; bj < 2; ++bj)
-#ifdef SBVR_GEMM_HACK_NOMFMA
-                    acc[bi][bj][0] += static_cast<float>(af[bi][0] + bf[bj][1]);
-#else
-                    acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[bi], bf[bj], acc[bi][bj], 0, 0, 0);
-#endif
+                    bf[bj] = *reinterpret_cast<const v8h *>(Bt + (brow + 32 * bj) * 128 + coff);
+#pragma unroll
+                for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+                    for (int bj = 0; bj < 2; ++bj)
+                        acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[bi], bf[bj], acc[bi][bj], 0, 0, 0);
+            }
         }
         __syncthreads();
     }
@@ -842,23 +875,38 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
 bool gemm_path_ok(int M, int N, int K, int S, int G)
 {
     return M > kMaxM && K % kGemmBK == 0 && G % kGemmBK == 0 && (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) &&
-           static_cast<double>(K / 32) * N * S < 2147483648.0;
+           static_cast<double>(K / 32) * N * S < 2147483648.0 && static_cast<double>(M) * K < 2147483648.0;
 }
 
 hipError_t launch_gemm(int S, const GemmArgs &a, hipStream_t st)
 {
     const dim3 grid(static_cast<unsigned>((a.N + kGemmBN - 1) / kGemmBN), static_cast<unsigned>((a.M + kGemmBM - 1) / kGemmBM));
     const dim3 block(kGemmThreads);
+    const size_t lds = 2 * (kGemmATile + kGemmBTile);      // 96 KiB: above the 64 KiB a kernel gets without asking
+#define SBVR_GEMM_LAUNCH(SS)                                                                                   \
+    {                                                                                                          \
+        static bool raised = false;                                                                            \
+        if (!raised) {                                                                                         \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sbvr_gemm_mfma_kernel<SS>), \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+            if (e != hipSuccess)                                                                               \
+                return e;                                                                                      \
+            raised = true;                                                                                     \
+        }                                                                                                      \
+        hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<SS>, grid, block, lds, st, a);                                \
+    }                                                                                                          \
+    break
     switch (S) {
-    case 4: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<4>, grid, block, 0, st, a); break;
+    case 4: SBVR_GEMM_LAUNCH(4);
 #ifndef SBVR_FAST_BUILD
-    case 2: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<2>, grid, block, 0, st, a); break;
-    case 3: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<3>, grid, block, 0, st, a); break;
-    case 6: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<6>, grid, block, 0, st, a); break;
-    case 8: hipLaunchKernelGGL(sbvr_gemm_mfma_kernel<8>, grid, block, 0, st, a); break;
+    case 2: SBVR_GEMM_LAUNCH(2);
+    case 3: SBVR_GEMM_LAUNCH(3);
+    case 6: SBVR_GEMM_LAUNCH(6);
+    case 8: SBVR_GEMM_LAUNCH(8);
 #endif
     default: return hipErrorInvalidConfiguration;
     }
+#undef SBVR_GEMM_LAUNCH
     return hipGetLastError();
 }
 
