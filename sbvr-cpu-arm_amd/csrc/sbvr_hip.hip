@@ -739,8 +739,7 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
                     cr[j] = cp[2 * j];
             }
             line[0] = line[1];
-            if (t + 2 < steps)
-                line[1] = load_line(t + 2);
+            line[1] = load_line(min(t + 2, steps - 1));
         };
         // one register set -> LDS buffers t % 2
         auto produce = [&](int t, const v4u (&ar)[8], const uint32_t (&wr)[S], const uint32_t (&cr)[CW]) __attribute__((always_inline)) {
@@ -778,36 +777,31 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
                 *reinterpret_cast<v4u *>(At + a_dst + 4096 * i) = ar[i];
         };
 #define SBVR_SET(n) areg##n, wreg##n, creg##n
+        // Requests are never conditional (beyond the last tile they repeat it): after a
+        // branch that may or may not have issued loads, the wait for an older set would
+        // have to assume it had not, and wait for everything.
+        const int last = steps - 1;
         line[0] = load_line(0);
-        if (steps > 1)
-            line[1] = load_line(1);
+        line[1] = load_line(min(1, last));
         request(0, SBVR_SET(0));
-        if (steps > 1)
-            request(1, SBVR_SET(1));
-        if (steps > 2)
-            request(2, SBVR_SET(2));
+        request(min(1, last), SBVR_SET(1));
+        request(min(2, last), SBVR_SET(2));
         produce(0, SBVR_SET(0));
         __syncthreads();
         // step i: the consumers read tile i; tile i+1 goes to the other buffers, tile i+3 is requested
         for (int r = 0; r < rounds; ++r) {
             const int i = 3 * r;
-            if (i + 1 < steps) {
-                if (i + 3 < steps)
-                    request(i + 3, SBVR_SET(0));
+            request(min(i + 3, last), SBVR_SET(0));
+            if (i + 1 < steps)
                 produce(i + 1, SBVR_SET(1));
-            }
             __syncthreads();
-            if (i + 2 < steps) {
-                if (i + 4 < steps)
-                    request(i + 4, SBVR_SET(1));
+            request(min(i + 4, last), SBVR_SET(1));
+            if (i + 2 < steps)
                 produce(i + 2, SBVR_SET(2));
-            }
             __syncthreads();
-            if (i + 3 < steps) {
-                if (i + 5 < steps)
-                    request(i + 5, SBVR_SET(2));
+            request(min(i + 5, last), SBVR_SET(2));
+            if (i + 3 < steps)
                 produce(i + 3, SBVR_SET(0));
-            }
             __syncthreads();
         }
 #undef SBVR_SET
