@@ -139,6 +139,86 @@ def decode_leg(prompt_tokens=128, new_tokens=128):
     return out
 
 
+def _graph_time(fn, iters):
+    """Seconds per call of fn(i), i = 0..iters-1, recorded into one HIP graph and replayed (best of 3)."""
+    import torch
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        fn(0)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(iters):
+                fn(i)
+        graph.replay()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            graph.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e-3 / iters
+            best = t if best is None else min(best, t)
+    return best
+
+
+def sweep_leg():
+    """The other decode configurations of the reference's benchmark plan: every linear of a
+    Llama-3-8B layer at batch 1, and gate / down at batch 1..16 with 2, 3 and 4 planes.
+    Weights rotate through enough copies to exceed the 256 MB Infinity Cache."""
+    import torch
+    from sbvr import synth, hip
+    dev = torch.device("cuda:0")
+    rows = []
+
+    def one(n, k, s, m, tag):
+        per = n * k * s // 8
+        copies = max(2, min(16, int(600e6 // per)))
+        ws = [tuple(t.to(dev) for t in synth.random_encoding(n, k, s, GROUP, LINES, seed=c)) for c in range(copies)]
+        x = torch.randn((m, k), generator=torch.Generator().manual_seed(5)).to(torch.float16).to(dev)
+        out = torch.empty((m, n), dtype=torch.float16, device=dev)
+        t = _graph_time(lambda i: hip._sbvr_linear_f16(x, *ws[i % copies], None, GROUP, out=out), 100)
+        nbytes = algorithmic_bytes(n, k, s, GROUP, LINES, m)
+        rows.append({"linear": tag, "N": n, "K": k, "S": s, "M": m, "us": round(t * 1e6, 2),
+                     "GBps": round(nbytes / t / 1e9, 1), "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4)})
+        del ws
+        torch.cuda.empty_cache()
+
+    for tag, n, k in (("q/o", 4096, 4096), ("k/v", 1024, 4096), ("q|k|v", 6144, 4096), ("gate/up", 14336, 4096),
+                      ("gate|up", 28672, 4096), ("down", 4096, 14336)):
+        one(n, k, 4, 1, tag)
+    for tag, n, k in (("gate", 14336, 4096), ("down", 4096, 14336)):
+        for s in (2, 3, 4):
+            for m in (1, 2, 4, 8, 16):
+                if not (s == 4 and m == 1):
+                    one(n, k, s, m, tag)
+    return rows
+
+
+def prefill_leg():
+    """Prefill GEMM at the 70B-width linears, S=4, G=128: dense-equivalent TFLOP/s against
+    the fp16 MFMA peak."""
+    import torch
+    from sbvr import synth, hip
+    dev = torch.device("cuda:0")
+    rows = []
+    for n, k in ((28672, 8192), (8192, 28672)):
+        w = tuple(t.to(dev) for t in synth.random_encoding(n, k, NUM_SUMS, GROUP, LINES, seed=1))
+        for m in (256, 512, 1024, 2048):
+            x = torch.randn((m, k), generator=torch.Generator().manual_seed(6)).to(torch.float16).to(dev)
+            out = torch.empty((m, n), dtype=torch.float16, device=dev)
+            t = _graph_time(lambda i: hip._sbvr_linear_f16(x, *w, None, GROUP, out=out), 5)
+            flops = 2.0 * m * n * k
+            rows.append({"N": n, "K": k, "M": m, "us": round(t * 1e6, 1), "TFLOPs": round(flops / t / 1e12, 1),
+                         "frac_of_fp16_mfma_peak": round(flops / t / 1e12 / 2500.0, 4)})
+        del w
+        torch.cuda.empty_cache()
+    return rows
+
+
 def cpu_decode_estimate(threads, per_shape_budget_s=1.5):
     """Time of the linears of one token on the host: the reference CPU kernel (x86 port)
     on each of the seven layer shapes, times 32 layers.  Excludes head, norms and attention."""
@@ -216,6 +296,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the 8B decode tokens/s leg")
     ap.add_argument("--decode-only", action="store_true", help="run only the 8B decode leg and print its figures")
+    ap.add_argument("--sweep", action="store_true",
+                    help="run only the layer-shape / batch / plane-count sweep of the decode kernel and print it")
+    ap.add_argument("--prefill", action="store_true", help="run only the prefill GEMM sizes and print them")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size kernel that "
                          "hardware byte counters are scaled by when profiling")
@@ -225,6 +308,12 @@ def main():
 
     if a.decode_only:
         print(json.dumps({"metric": "8B decode tokens/s", "decode": decode_leg()}))
+        return
+    if a.sweep:
+        print(json.dumps({"metric": "SBVR decode linears, us and GB/s of algorithmic bytes", "sweep": sweep_leg()}))
+        return
+    if a.prefill:
+        print(json.dumps({"metric": "SBVR prefill GEMM, dense-equivalent TFLOP/s", "prefill": prefill_leg()}))
         return
     if a.calibrate_copy:
         import torch

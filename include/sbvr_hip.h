@@ -60,7 +60,12 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  *               sbvr/kernels/sbvr_kernel.cu:555-559 does
  *   out         (M, N)      fp16
  * fp32 accumulation, one rounding to fp16.  K must be a multiple of G and G of
- * 32.  The reference has no kernel of exactly this form (its fp16-activation
+ * 32.  M <= 16 takes the decode kernel (plane sums on the matrix cores, exact
+ * fp16 activations); larger M takes the prefill kernel, which decodes weight
+ * tiles to fp16 first (each decoded weight an fp16 sum of its coefficients, as
+ * decode() of sbvr/core.py:927-949 rounds weights to fp16) and needs K and G to
+ * be multiples of 64; other shapes fall back to the portable kernel.
+ * The reference has no kernel of exactly this form (its fp16-activation
  * kernels, sbvr_kernel.cu:121-359 behind sbvr_ops.cpp:79-120, want the
  * trans=True layout); this is the operator its models/sbvr_llama.py:86-87
  * SBVRLinear.forward stands for.

@@ -7,11 +7,11 @@
 //   * a 32-bit plane word becomes four dwords of fp4 (e2m1) values with one AND
 //     (or shift+AND) each: nibble q of dword t carries bit 4q+t of the word as
 //     0.5, 1.0 or 2.0;
-//   * the fp16 activations of one 128-element sub-group are written, once per
-//     workgroup, as three fp8 (e4m3) terms h1 + h2 + h3/256 = x * 2^e * f_t, which
-//     reproduce the fp16 value exactly (4 significant bits each, the third taken
-//     from the residual scaled by 256), in the register image of the A operand;
-//     the per-position factor f_t undoes the 0.5/1/2 of the B nibbles, 2^e is a
+//   * the fp16 activations of one 128-element sub-group are written as three
+//     fp8 (e4m3) terms h1 + h2 + h3/256 = x * 2^e * f_t, which reproduce the
+//     fp16 value exactly (4 significant bits each, the third taken from the
+//     residual scaled by 256), in the register image of the A operand; the
+//     per-position factor f_t undoes the 0.5/1/2 of the B nibbles, 2^e is a
 //     power of two per (row, sub-group);
 //   * v_mfma_f32_16x16x128_f8f6f4 (A fp8, B fp4) then yields, for 16 columns
 //     and one plane, the three partial plane sums per batch row; they are added,
@@ -19,10 +19,17 @@
 // The packed layout of the reference (sbvr/core.py:724-731, 782-805) is read as
 // it is: a lane loads the S plane words of one (word, column) pair with one
 // vector load, 16 neighbouring columns give 256 contiguous bytes.
+// Work split: a workgroup owns 16*CT columns, its waves split K and add their
+// partial results in LDS in a fixed order; when N alone does not give enough
+// workgroups, K is also split across workgroups, whose partial sums meet in
+// 64-bit fixed-point accumulators (exact, so the result does not depend on
+// the order of arrival).
 //
-// Work split: a workgroup owns 64*CT columns and SP sub-groups of K; K is split
-// over workgroups, partial sums go to a workspace and the last workgroup to
-// finish a column tile adds them in a fixed order (deterministic result).
+// Prefill path (M > 16), sbvr_gemm_mfma_kernel: weights decoded to fp16 tiles
+// in LDS, fp16 MFMA, fp32 accumulation.
+//
+// Portable kernels (any shape, one thread per output) back both, and serve the
+// trans=True and both-operands-encoded forms of the reference's operators.
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdint.h>
