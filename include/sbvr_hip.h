@@ -60,8 +60,8 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  *               sbvr/kernels/sbvr_kernel.cu:555-559 does
  *   out         (M, N)      fp16
  * fp32 accumulation, one rounding to fp16.  K must be a multiple of G and G of
- * 32.  M <= 16 takes the decode kernel (plane sums on the matrix cores, exact
- * fp16 activations); larger M takes the prefill kernel, which decodes weight
+ * 32.  M <= 4 (M <= 16 with flags bit 1) takes the decode kernel (plane sums on
+ * the matrix cores, exact fp16 activations); larger M takes the prefill kernels, which decodes weight
  * tiles to fp16 first (each decoded weight an fp16 sum of its coefficients, as
  * decode() of sbvr/core.py:927-949 rounds weights to fp16) and needs K and G to
  * be multiples of 64; other shapes fall back to the portable kernel.
@@ -69,7 +69,10 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  * kernels, sbvr_kernel.cu:121-359 behind sbvr_ops.cpp:79-120, want the
  * trans=True layout); this is the operator its models/sbvr_llama.py:86-87
  * SBVRLinear.forward stands for.
- * flags: bit 0 forces the portable kernel (one thread per output).
+ * flags: bit 0 forces the portable kernel (one thread per output); bit 1 keeps
+ * the decode kernel for 5..16 rows, where the default is a 32-row MFMA kernel
+ * that decodes weights to fp16 like the prefill kernel (faster there, and with
+ * the prefill kernel's rounding).
  */
 int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_idx,
                         int idx_bytes, const void *coeff_cache, const void *bias,

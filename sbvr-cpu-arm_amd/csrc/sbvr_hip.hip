@@ -873,6 +873,212 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
     }
 }
 
+// ------------------------------------------------- MFMA, 5 to 32 batch rows
+
+// Between the decode kernel (whose cost grows with the batch rows: each needs
+// its own fp8 A operands) and the prefill kernel (256-row tiles) sits a kernel
+// for up to 32 rows: v_mfma_f32_32x32x16_f16 with the batch rows as the 32 rows
+// of A, read from global memory as they are, and 32 columns of decoded weights
+// as B.  A wave walks a range of K one 32-bit word (two MFMAs) at a time; lane
+// (column j, half h) decodes bits 8h..8h+7 and 16+8h..16+8h+7 of the word, two
+// elements (k, k+16) per packed fp16 operation as in the prefill kernel, which
+// are exactly its B elements of the two MFMAs.  No LDS on the way; the 8 waves
+// of a workgroup split K and add their 32 x 32 partial results in LDS at the
+// end.  Bound by the decode arithmetic (about 7.5 VALU operations per weight),
+// not by the batch size.
+constexpr int kRowsMax = 32, kRowsWaves = 8, kRowsBlock = 2;
+
+struct RowsArgs {
+    const uint16_t *x;
+    const uint32_t *bvr;
+    const void *idx;
+    const uint16_t *cache;
+    const uint16_t *bias;
+    uint16_t *out;
+    int M, N, K, L;
+    int words_per_group;   // G / 32
+    int words_per_wave;    // a multiple of kRowsBlock
+    int idx16;
+};
+
+template <int S>
+__global__ void __launch_bounds__(64 * kRowsWaves)
+sbvr_gemm_rows32_kernel(const RowsArgs a)
+{
+    __shared__ float red[kRowsWaves][16][64];
+    constexpr int CW = (S + 1) / 2;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int N = a.N, K = a.K, M = a.M;
+    const int j = lane & 31, h = lane >> 5;
+    const int n = blockIdx.x * 32 + j, n_ld = min(n, N - 1);
+    const int words = K / 32;
+    const int w_begin = wave * a.words_per_wave, w_end = min(words, w_begin + a.words_per_wave);
+    const bool row_ok = j < M;                        // lane's batch row for the A operand is j as well
+    const uint16_t *xrow = a.x + static_cast<size_t>(min(j, M - 1)) * K + 8 * h;
+
+    struct Block {
+        v4u planes[kRowsBlock];      // S <= 4 words used directly; more planes: see below
+        uint32_t more[kRowsBlock][S > 4 ? S - 4 : 1];
+        v4u xa[kRowsBlock][2];
+        uint32_t c[kRowsBlock][CW];
+    };
+    auto load_lines = [&](int w0, int (&line)[kRowsBlock]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kRowsBlock; ++i) {
+            const int w = min(w0 + i, words - 1);
+            const size_t at = static_cast<size_t>(w / a.words_per_group) * N + n_ld;
+            const int v = a.idx16 ? static_cast<int>(static_cast<const uint16_t *>(a.idx)[at])
+                                  : static_cast<int>(static_cast<const uint8_t *>(a.idx)[at]);
+            line[i] = min(v, a.L - 1);
+        }
+    };
+    auto load_block = [&](int w0, Block &b, const int (&line)[kRowsBlock]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kRowsBlock; ++i) {
+            const int w = min(w0 + i, words - 1);        // beyond the range: repeats the last word, never used
+            const uint32_t *wp = a.bvr + (static_cast<size_t>(w) * N + n_ld) * S;
+            const Planes<S> pl = load_planes<S>(wp);
+#pragma unroll
+            for (int q = 0; q < S; ++q) {
+                if (q < 4)
+                    b.planes[i][q] = pl.w[q];
+                else
+                    b.more[i][q - 4] = pl.w[q];
+            }
+            b.xa[i][0] = v4u{0u, 0u, 0u, 0u};
+            b.xa[i][1] = v4u{0u, 0u, 0u, 0u};
+            if (row_ok) {
+                b.xa[i][0] = *reinterpret_cast<const v4u *>(xrow + 32 * w);
+                b.xa[i][1] = *reinterpret_cast<const v4u *>(xrow + 32 * w + 16);
+            }
+            const uint16_t *cp = a.cache + static_cast<size_t>(line[i]) * S;
+#pragma unroll
+            for (int q = 0; q < CW; ++q) {
+                if (S % 2 == 0 || 2 * q + 1 < S)
+                    b.c[i][q] = static_cast<uint32_t>(cp[2 * q]) | (static_cast<uint32_t>(cp[2 * q + 1]) << 16);
+                else
+                    b.c[i][q] = cp[2 * q];
+            }
+        }
+    };
+
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        acc[r] = 0.f;
+
+    auto compute = [&](int w0, const Block &b) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kRowsBlock; ++i) {
+            if (w0 + i >= w_end)          // wave-uniform
+                break;
+            uint32_t wsh[S], cbits[S];
+#pragma unroll
+            for (int q = 0; q < S; ++q) {
+                const uint32_t word = q < 4 ? b.planes[i][q < 4 ? q : 0] : b.more[i][q < 4 ? 0 : q - 4];
+                wsh[q] = word >> (8 * h);
+                cbits[q] = q & 1 ? b.c[i][q / 2] >> 16 : b.c[i][q / 2] & 0xffffu;
+            }
+            uint32_t pr[8];               // pr[e] = {w[8h+e], w[16+8h+e]}
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v2h v = __builtin_bit_cast(v2h, __umul24((wsh[0] >> e) & 0x00010001u, cbits[0]));
+#pragma unroll
+                for (int q = 1; q < S; ++q)
+                    v = v + __builtin_bit_cast(v2h, __umul24((wsh[q] >> e) & 0x00010001u, cbits[q]));
+                pr[e] = __builtin_bit_cast(uint32_t, v);
+            }
+            v4u b0, b1;
+            b0.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x05040100u); b1.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x07060302u);
+            b0.y = __builtin_amdgcn_perm(pr[3], pr[2], 0x05040100u); b1.y = __builtin_amdgcn_perm(pr[3], pr[2], 0x07060302u);
+            b0.z = __builtin_amdgcn_perm(pr[5], pr[4], 0x05040100u); b1.z = __builtin_amdgcn_perm(pr[5], pr[4], 0x07060302u);
+            b0.w = __builtin_amdgcn_perm(pr[7], pr[6], 0x05040100u); b1.w = __builtin_amdgcn_perm(pr[7], pr[6], 0x07060302u);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, b.xa[i][0]), __builtin_bit_cast(v8h, b0), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, b.xa[i][1]), __builtin_bit_cast(v8h, b1), acc, 0, 0, 0);
+        }
+    };
+
+    // two register blocks in turn; the line indices run one block further ahead
+    // (loads are never conditional, see the prefill kernel)
+    Block b0, b1;
+    int line[kRowsBlock];
+    load_lines(w_begin, line);
+    load_block(w_begin, b0, line);
+    load_lines(w_begin + kRowsBlock, line);
+    for (int w0 = w_begin; w0 < w_end; w0 += 2 * kRowsBlock) {
+        load_block(w0 + kRowsBlock, b1, line);
+        load_lines(w0 + 2 * kRowsBlock, line);
+        compute(w0, b0);
+        load_block(w0 + 2 * kRowsBlock, b0, line);
+        load_lines(w0 + 3 * kRowsBlock, line);
+        compute(w0 + kRowsBlock, b1);
+    }
+
+    // ---- partial results meet in LDS; D[i][jj] sits in lane jj + 32*((i/4)%2), register (i%4) + 4*(i/8)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        red[wave][r][lane] = acc[r];
+    __syncthreads();
+    if (n >= N)
+        return;
+    const uint16_t bias = a.bias ? a.bias[n] : 0;
+#pragma unroll
+    for (int rr = 0; rr < 16 / kRowsWaves; ++rr) {
+        const int r = wave * (16 / kRowsWaves) + rr;
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < kRowsWaves; ++w)
+            total += red[w][r][lane];
+        const int m = 8 * (r >> 2) + 4 * h + (r & 3);
+        if (m < M) {
+            uint16_t v = f2h(total);
+            if (a.bias)
+                v = hadd(v, bias);
+            a.out[static_cast<size_t>(m) * N + n] = v;
+        }
+    }
+}
+
+bool rows32_path_ok(int M, int N, int K, int S, int G)
+{
+    return M > 4 && M <= kRowsMax && K % 32 == 0 && G % 32 == 0 && (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) &&
+           static_cast<double>(K / 32) * N * S < 2147483648.0;
+}
+
+// Measured on MI355X at the Llama-3-8B shapes: the 32-row kernel takes about the same
+// time for any batch up to 32 (24 us at 4096 -> 14336), the decode kernel 17 us at 8 rows
+// and 34 us at 16; with fewer than one 32-column workgroup per CU the 32-row kernel loses.
+bool rows32_preferred(int M, int N, int K, int S, int G, int cus)
+{
+    if (!rows32_path_ok(M, N, K, S, G))
+        return false;
+    if (M <= kMaxM && mfma_path_ok(M, N, K, S, G))
+        return M > 8 && (N + 31) / 32 >= cus;
+    return true;          // no decode kernel for this shape, or 17..32 rows
+}
+
+hipError_t launch_rows32(int S, RowsArgs a, hipStream_t st)
+{
+    const int words = a.K / 32;
+    int wpw = (words + kRowsWaves - 1) / kRowsWaves;
+    wpw = (wpw + kRowsBlock - 1) / kRowsBlock * kRowsBlock;
+    a.words_per_wave = wpw;
+    const dim3 grid(static_cast<unsigned>((a.N + 31) / 32)), block(64 * kRowsWaves);
+    switch (S) {
+    case 4: hipLaunchKernelGGL(sbvr_gemm_rows32_kernel<4>, grid, block, 0, st, a); break;
+#ifndef SBVR_FAST_BUILD
+    case 2: hipLaunchKernelGGL(sbvr_gemm_rows32_kernel<2>, grid, block, 0, st, a); break;
+    case 3: hipLaunchKernelGGL(sbvr_gemm_rows32_kernel<3>, grid, block, 0, st, a); break;
+    case 6: hipLaunchKernelGGL(sbvr_gemm_rows32_kernel<6>, grid, block, 0, st, a); break;
+    case 8: hipLaunchKernelGGL(sbvr_gemm_rows32_kernel<8>, grid, block, 0, st, a); break;
+#endif
+    default: return hipErrorInvalidConfiguration;
+    }
+    return hipGetLastError();
+}
+
 bool gemm_path_ok(int M, int N, int K, int S, int G)
 {
     return M > kMaxM && K % kGemmBK == 0 && G % kGemmBK == 0 && (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) &&
@@ -1053,6 +1259,22 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
 
     const bool aligned = reinterpret_cast<uintptr_t>(bvr) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(coeff_cache) % 16 == 0;
+    if (!(flags & 3) && aligned && rows32_preferred(M, N, K, S, G, current_cus()) && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        RowsArgs r{};
+        r.x = static_cast<const uint16_t *>(x);
+        r.bvr = bvr;
+        r.idx = coeff_idx;
+        r.cache = static_cast<const uint16_t *>(coeff_cache);
+        r.bias = static_cast<const uint16_t *>(bias);
+        r.out = static_cast<uint16_t *>(out);
+        r.M = M; r.N = N; r.K = K; r.L = L;
+        r.words_per_group = G / 32;
+        r.idx16 = idx_bytes == 2;
+        const hipError_t e = launch_rows32(S, r, st);
+        if (e != hipSuccess)
+            return fail(SBVR_HIP_ELAUNCH, "rows32 launch: %s", hipGetErrorString(e));
+        return SBVR_HIP_OK;
+    }
     if (!(flags & 1) && aligned && mfma_path_ok(M, N, K, S, G)) {
         const GemvPlan p = plan_gemv(M, N, K, S, current_cus());
         if (p.CT > 0) {

@@ -67,6 +67,31 @@ def test_two_tiles_each_way(oracle):
     run_case(oracle, 384, 1024, 4, 128, 520, 256, seed=43)
 
 
+@pytest.mark.parametrize("M", [5, 8, 16, 31, 32])
+def test_rows32_kernel_rows(oracle, M):
+    """5..32 rows: 32-row MFMA kernel with the weights decoded in registers."""
+    run_case(oracle, 256, 512, 4, 128, M, 256, seed=70 + M)
+
+
+@pytest.mark.parametrize("S,G", [(2, 128), (3, 128), (4, 32), (4, 64), (4, 256), (6, 128), (8, 128)])
+def test_rows32_kernel_planes_groups(oracle, S, G):
+    run_case(oracle, 96, 768, S, G, 12, 200, seed=80 + S + G)
+
+
+@pytest.mark.parametrize("N,K", [(16, 256), (100, 160), (1000, 96), (130, 2048)])
+def test_rows32_kernel_ragged(oracle, N, K):
+    run_case(oracle, N, K, 4, 32, 7, 64, seed=90 + N)
+
+
+def test_rows32_kernel_u16_index_and_bias(oracle):
+    run_case(oracle, 320, 768, 4, 128, 9, 3000, seed=95)
+    run_case(oracle, 320, 768, 3, 128, 16, 256, seed=96, bias=True)
+
+
+def test_rows32_kernel_gate_shape(oracle):
+    run_case(oracle, 14336, 4096, 4, 128, 16, 256, seed=97)
+
+
 def test_matches_decode_path_rows():
     """The same rows through the decode path (16 at a time) and the prefill path."""
     import sbvr

@@ -60,7 +60,9 @@ def test_small_m1(oracle, S, G):
 
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 16])
 def test_batch(oracle, M):
-    run_case(oracle, 512, 1024, 4, 128, M, 256, seed=3)
+    # flags bit 1 keeps the decode kernel above 4 rows (the default there is the 32-row kernel,
+    # which has its own tests and tolerance in test_gpu_gemm_parity.py)
+    run_case(oracle, 512, 1024, 4, 128, M, 256, seed=3, flags=2 if M > 4 else 0)
 
 
 def test_u16_index(oracle):
@@ -91,7 +93,7 @@ def test_llama_shapes(oracle, N, K):
 @pytest.mark.parametrize("S", [2, 3, 4])
 @pytest.mark.parametrize("M", [2, 16])
 def test_sweep_gate(oracle, S, M):
-    run_case(oracle, 14336, 4096, S, 128, M, 256, seed=12)
+    run_case(oracle, 14336, 4096, S, 128, M, 256, seed=12, flags=2 if M > 4 else 0)
 
 
 def test_portable_kernel(oracle):
