@@ -98,6 +98,29 @@ def test_small_decoder_matches_dense(oracle, graph):
             assert ref[p][picked[p]] >= ref[p].max() - 2e-2 * np.abs(ref[p]).max()
 
 
+def test_long_cache_uses_looped_attention(oracle):
+    """A cache longer than the all-in-registers attention variant holds (512 positions at head_dim 64)."""
+    import torch
+    from sbvr.decoder import LlamaShape, SbvrLlamaDecoder
+
+    shape = LlamaShape(hidden=128, layers=1, heads=2, kv_heads=1, head_dim=64, ffn=256, vocab=300)
+    dec = SbvrLlamaDecoder(shape, "cuda:0", lines=32, max_seq=600, seed=9)
+    for layer in dec.layers:
+        for k in ("qkv", "o", "gate_up", "down"):
+            layer[k].cache.mul_(2.0)
+    tokens = [int(t) for t in torch.randint(0, 300, (40,), generator=torch.Generator().manual_seed(2))]
+    dec.reset()
+    got = []
+    with torch.cuda.stream(dec.stream):
+        for t in tokens:
+            dec.tok.fill_(t)
+            got.append(dec.step().float().cpu().numpy()[0])
+    ref = dense_reference(dec, oracle, tokens)
+    for p in (0, 1, 17, 39):
+        err = np.abs(got[p] - ref[p]).max() / np.abs(ref[p]).max()
+        assert err < 2e-2, f"step {p}: logits differ by {err:.3e} of the largest"
+
+
 def test_generate_is_repeatable():
     import torch
     from sbvr.decoder import LlamaShape, SbvrLlamaDecoder
