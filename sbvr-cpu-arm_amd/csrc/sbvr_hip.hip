@@ -720,11 +720,13 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
         uint32_t creg0[CW], creg1[CW], creg2[CW];
         int line[2] = {0, 0};       // line index of the tile to be requested next, and of the one after
 
+        // (two byte loads whatever the index width: a branch between a 16-bit and an 8-bit load
+        // inside the loop would make every later wait a wait for all loads)
         auto load_line = [&](int t) __attribute__((always_inline)) -> int {
-            const size_t at = static_cast<size_t>(t / a.steps_per_group) * N + n_ld;
-            const int v = a.idx16 ? static_cast<int>(static_cast<const uint16_t *>(a.idx)[at])
-                                  : static_cast<int>(static_cast<const uint8_t *>(a.idx)[at]);
-            return min(v, a.L - 1);
+            const size_t at = (static_cast<size_t>(t / a.steps_per_group) * N + n_ld) << a.idx16;
+            const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
+            const int lo = ib[at], hi = ib[at + a.idx16];
+            return min(a.idx16 ? lo | (hi << 8) : lo, a.L - 1);
         };
         // global loads of tile t into one register set
         auto request = [&](int t, v4u (&ar)[8], uint32_t (&wr)[S], uint32_t (&cr)[CW]) __attribute__((always_inline)) {
@@ -798,17 +800,16 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
         // step i: the consumers read tile i; tile i+1 goes to the other buffers, tile i+3 is requested
         for (int r = 0; r < rounds; ++r) {
             const int i = 3 * r;
+            // (tiles beyond the last are produced too, from repeated loads, into buffers nobody reads:
+            // a loop body without branches keeps the waits of the three register sets apart)
             request(min(i + 3, last), SBVR_SET(0));
-            if (i + 1 < steps)
-                produce(i + 1, SBVR_SET(1));
+            produce(i + 1, SBVR_SET(1));
             __syncthreads();
             request(min(i + 4, last), SBVR_SET(1));
-            if (i + 2 < steps)
-                produce(i + 2, SBVR_SET(2));
+            produce(i + 2, SBVR_SET(2));
             __syncthreads();
             request(min(i + 5, last), SBVR_SET(2));
-            if (i + 3 < steps)
-                produce(i + 3, SBVR_SET(0));
+            produce(i + 3, SBVR_SET(0));
             __syncthreads();
         }
 #undef SBVR_SET
@@ -828,25 +829,36 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
     const int arow = wm * 128 + (lane & 31), brow = wn * 64 + (lane & 31);      // + 32 bi / bj: same row & 7
     const int rsw = lane & 7, chi = lane >> 5;
     __syncthreads();
+    // operand registers of two k-slices in turn: the reads of slice s+1 are issued before the MFMAs of slice s
+    auto read_slice = [&](const unsigned char *At, const unsigned char *Bt, int ks, v8h (&af)[4], v8h (&bf)[2])
+                          __attribute__((always_inline)) {
+        const int coff = ((2 * ks + chi) ^ rsw) << 4;
+#pragma unroll
+        for (int bi = 0; bi < 4; ++bi)
+            af[bi] = *reinterpret_cast<const v8h *>(At + (arow + 32 * bi) * 128 + coff);
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+            bf[bj] = *reinterpret_cast<const v8h *>(Bt + (brow + 32 * bj) * 128 + coff);
+    };
+    auto mfma_slice = [&](const v8h (&af)[4], const v8h (&bf)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+            for (int bj = 0; bj < 2; ++bj)
+                acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[bi], bf[bj], acc[bi][bj], 0, 0, 0);
+    };
     for (int i = 0; i < 3 * rounds; ++i) {
         if (i < steps) {
             const unsigned char *At = As + (i & 1) * kGemmATile, *Bt = Bs + (i & 1) * kGemmBTile;
-#pragma unroll
-            for (int ks = 0; ks < kGemmBK / 16; ++ks) {
-                const int coff = ((2 * ks + chi) ^ rsw) << 4;
-                v8h af[4], bf[2];
-#pragma unroll
-                for (int bi = 0; bi < 4; ++bi)
-                    af[bi] = *reinterpret_cast<const v8h *>(At + (arow + 32 * bi) * 128 + coff);
-#pragma unroll
-                for (int bj = 0; bj < 2; ++bj)
-                    bf[bj] = *reinterpret_cast<const v8h *>(Bt + (brow + 32 * bj) * 128 + coff);
-#pragma unroll
-                for (int bi = 0; bi < 4; ++bi)
-#pragma unroll
-                    for (int bj = 0; bj < 2; ++bj)
-                        acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[bi], bf[bj], acc[bi][bj], 0, 0, 0);
-            }
+            v8h af0[4], bf0[2], af1[4], bf1[2];
+            read_slice(At, Bt, 0, af0, bf0);
+            read_slice(At, Bt, 1, af1, bf1);
+            mfma_slice(af0, bf0);
+            read_slice(At, Bt, 2, af0, bf0);
+            mfma_slice(af1, bf1);
+            read_slice(At, Bt, 3, af1, bf1);
+            mfma_slice(af0, bf0);
+            mfma_slice(af1, bf1);
         }
         __syncthreads();
     }
@@ -928,10 +940,10 @@ sbvr_gemm_rows32_kernel(const RowsArgs a)
 #pragma unroll
         for (int i = 0; i < kRowsBlock; ++i) {
             const int w = min(w0 + i, words - 1);
-            const size_t at = static_cast<size_t>(w / a.words_per_group) * N + n_ld;
-            const int v = a.idx16 ? static_cast<int>(static_cast<const uint16_t *>(a.idx)[at])
-                                  : static_cast<int>(static_cast<const uint8_t *>(a.idx)[at]);
-            line[i] = min(v, a.L - 1);
+            const size_t at = (static_cast<size_t>(w / a.words_per_group) * N + n_ld) << a.idx16;
+            const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
+            const int lo = ib[at], hi = ib[at + a.idx16];      // two byte loads whatever the width: no branch
+            line[i] = min(a.idx16 ? lo | (hi << 8) : lo, a.L - 1);
         }
     };
     auto load_block = [&](int w0, Block &b, const int (&line)[kRowsBlock]) __attribute__((always_inline)) {
