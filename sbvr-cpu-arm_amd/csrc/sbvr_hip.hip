@@ -1208,6 +1208,134 @@ sbvr_mm_T_kernel(const uint32_t *__restrict__ l_bvr, const void *__restrict__ l_
     out[o] = res;
 }
 
+// Both operands encoded (the form the reference's kernels compute, sbvr_kernel.cu:464-562
+// and sbvr_kernel.cpp:251-399): out[m,n] = sum_g sum_{l,r} popcount_g(L_l & R_r) a_l b_r.
+// Lane = column, so a wave reads 64 * SR consecutive plane words per word of K (coalesced)
+// while the left operand's words and coefficients are wave-uniform (scalar loads).  The
+// waves of a workgroup split the groups of K and meet in LDS; blockIdx.y is the left row.
+// Popcounts are exact integers per group; coefficients are applied in fp32.
+constexpr int kPopcWaves = 8, kPopcChunk = 8;      // words of K whose plane words a lane holds at once
+
+template <int SL, int SR>
+__global__ void __launch_bounds__(64 * kPopcWaves)
+sbvr_mm_T_popc_kernel(const uint32_t *__restrict__ l_bvr, const uint8_t *__restrict__ l_idx, int l_idx16,
+                      const uint16_t *__restrict__ l_cache, const uint32_t *__restrict__ r_bvr,
+                      const uint8_t *__restrict__ r_idx, int r_idx16, const uint16_t *__restrict__ r_cache,
+                      const uint16_t *__restrict__ bias, uint16_t *__restrict__ out,
+                      int M, int N, int K, int wpg, int Ll, int Lr)
+{
+    __shared__ float red[kPopcWaves][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int m = blockIdx.y;
+    const int n = blockIdx.x * 64 + lane, n_ld = min(n, N - 1);
+    const int words = K / 32;
+    const int chunks = (words + kPopcChunk - 1) / kPopcChunk;
+    const int cpw = (chunks + kPopcWaves - 1) / kPopcWaves;         // chunks per wave
+    const int c_begin = wave * cpw, c_end = min(chunks, c_begin + cpw);
+
+    auto load_chunk = [&](int c, uint32_t (&rw)[kPopcChunk][SR], int (&line)[kPopcChunk]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < kPopcChunk; ++i) {
+            const int w = min(c * kPopcChunk + i, words - 1);       // beyond K: repeats the last word, never used
+            const Planes<SR> pl = load_planes<SR>(r_bvr + (static_cast<size_t>(w) * N + n_ld) * SR);
+#pragma unroll
+            for (int r = 0; r < SR; ++r)
+                rw[i][r] = pl.w[r];
+            // one line index per group; read per word (same address within a group: cached)
+            const size_t at = (static_cast<size_t>(w / wpg) * N + n_ld) << r_idx16;
+            const int lo = r_idx[at], hi = r_idx[at + r_idx16];
+            line[i] = min(r_idx16 ? lo | (hi << 8) : lo, Lr - 1);
+        }
+    };
+
+    float acc = 0.f;
+    uint32_t rw0[kPopcChunk][SR], rw1[kPopcChunk][SR];
+    int ln0[kPopcChunk], ln1[kPopcChunk];
+    auto compute = [&](int c, const uint32_t (&rw)[kPopcChunk][SR], const int (&line)[kPopcChunk]) __attribute__((always_inline)) {
+        int cnt[SL][SR];
+#pragma unroll
+        for (int l = 0; l < SL; ++l)
+#pragma unroll
+            for (int r = 0; r < SR; ++r)
+                cnt[l][r] = 0;
+#pragma unroll
+        for (int i = 0; i < kPopcChunk; ++i) {
+            const int w = c * kPopcChunk + i;
+            if (w >= words)                                          // wave-uniform
+                break;
+            const uint32_t *lp = l_bvr + (static_cast<size_t>(w) * M + m) * SL;       // wave-uniform
+#pragma unroll
+            for (int l = 0; l < SL; ++l) {
+                const uint32_t lw = __builtin_amdgcn_readfirstlane(lp[l]);
+#pragma unroll
+                for (int r = 0; r < SR; ++r)
+                    cnt[l][r] += __builtin_popcount(lw & rw[i][r]);
+            }
+            if ((i + 1) % wpg == 0) {                                // wave-uniform: last word of its group
+                const size_t lat = (static_cast<size_t>(w / wpg) * M + m) << l_idx16;
+                const int llo = l_idx[lat], lhi = l_idx[lat + l_idx16];
+                const int lline = __builtin_amdgcn_readfirstlane(min(l_idx16 ? llo | (lhi << 8) : llo, Ll - 1));
+                const uint16_t *ca = l_cache + static_cast<size_t>(lline) * SL;
+                const uint16_t *cb = r_cache + static_cast<size_t>(line[i]) * SR;
+                float group = 0.f;
+#pragma unroll
+                for (int r = 0; r < SR; ++r) {
+                    float t = 0.f;
+#pragma unroll
+                    for (int l = 0; l < SL; ++l) {
+                        t = fmaf(static_cast<float>(cnt[l][r]), h2f(ca[l]), t);
+                        cnt[l][r] = 0;
+                    }
+                    group = fmaf(t, h2f(cb[r]), group);
+                }
+                acc += group;
+            }
+        }
+    };
+
+    if (c_begin < c_end) {
+        load_chunk(c_begin, rw0, ln0);
+        for (int c = c_begin; c < c_end; c += 2) {
+            load_chunk(min(c + 1, chunks - 1), rw1, ln1);
+            compute(c, rw0, ln0);
+            load_chunk(min(c + 2, chunks - 1), rw0, ln0);
+            if (c + 1 < c_end)
+                compute(c + 1, rw1, ln1);
+        }
+    }
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && n < N) {
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < kPopcWaves; ++w)
+            total += red[w][lane];
+        uint16_t res = f2h(total);
+        if (bias)
+            res = hadd(res, bias[n]);
+        out[static_cast<size_t>(m) * N + n] = res;
+    }
+}
+
+template <int SL>
+bool launch_mm_T_popc_sr(int Sr, dim3 grid, hipStream_t st, const uint32_t *l_bvr, const uint8_t *l_idx, int l16,
+                         const uint16_t *lc, const uint32_t *r_bvr, const uint8_t *r_idx, int r16, const uint16_t *rc,
+                         const uint16_t *b, uint16_t *o, int M, int N, int K, int wpg, int Ll, int Lr)
+{
+    const dim3 block(64 * kPopcWaves);
+#define SBVR_POPC(SR)                                                                                              \
+    hipLaunchKernelGGL((sbvr_mm_T_popc_kernel<SL, SR>), grid, block, 0, st, l_bvr, l_idx, l16, lc, r_bvr, r_idx, \
+                       r16, rc, b, o, M, N, K, wpg, Ll, Lr)
+    switch (Sr) {
+    case 2: SBVR_POPC(2); return true;
+    case 3: SBVR_POPC(3); return true;
+    case 4: SBVR_POPC(4); return true;
+    default: return false;
+    }
+#undef SBVR_POPC
+}
+
 } // namespace
 
 // ------------------------------------------------------------------- C ABI
@@ -1404,6 +1532,27 @@ int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_byte
     const uint16_t *lc = static_cast<const uint16_t *>(l_coeff_cache), *rc = static_cast<const uint16_t *>(r_coeff_cache);
     const uint16_t *b = static_cast<const uint16_t *>(bias);
     uint16_t *o = static_cast<uint16_t *>(out);
+    // few left rows (the reference's kernels are written for one): lane-per-column popcount kernel
+    const int wpg = G / 32;
+    if (M <= 64 && (wpg == 1 || wpg == 2 || wpg == 4 || wpg == 8) && Sl >= 2 && Sl <= 4 &&
+        reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0 && static_cast<double>(K / 32) * N * Sr < 2147483648.0) {
+        const dim3 pgrid(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(M));
+        const uint8_t *li = static_cast<const uint8_t *>(l_coeff_idx), *ri = static_cast<const uint8_t *>(r_coeff_idx);
+        const int l16 = l_idx_bytes == 2, r16 = r_idx_bytes == 2;
+        bool done = false;
+        if (Sl == 2)
+            done = launch_mm_T_popc_sr<2>(Sr, pgrid, st, l_bvr, li, l16, lc, r_bvr, ri, r16, rc, b, o, M, N, K, wpg, Ll, Lr);
+        else if (Sl == 3)
+            done = launch_mm_T_popc_sr<3>(Sr, pgrid, st, l_bvr, li, l16, lc, r_bvr, ri, r16, rc, b, o, M, N, K, wpg, Ll, Lr);
+        else
+            done = launch_mm_T_popc_sr<4>(Sr, pgrid, st, l_bvr, li, l16, lc, r_bvr, ri, r16, rc, b, o, M, N, K, wpg, Ll, Lr);
+        if (done) {
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess)
+                return fail(SBVR_HIP_ELAUNCH, "mm_T launch: %s", hipGetErrorString(e));
+            return SBVR_HIP_OK;
+        }
+    }
 #define SBVR_MM_LAUNCH(LT, RT)                                                                   \
     hipLaunchKernelGGL((sbvr_mm_T_kernel<LT, RT>), grid, block, 0, st, l_bvr, l_coeff_idx, lc,   \
                        r_bvr, r_coeff_idx, rc, b, o, M, N, K, Sl, Sr, G)

@@ -23,7 +23,11 @@ def _close(y, yd, ulps=2.0):
 
 
 @pytest.mark.parametrize("M,N,K,Sl,Sr,G,Ll,Lr", [(1, 64, 512, 4, 4, 256, 5, 9), (3, 40, 256, 2, 3, 128, 300, 7),
-                                                 (2, 33, 512, 8, 6, 256, 4, 400)])
+                                                 (2, 33, 512, 8, 6, 256, 4, 400),       # no popcount-kernel instance
+                                                 (1, 1000, 160, 4, 4, 32, 16, 256),     # 5 words: a partial chunk
+                                                 (1, 130, 4096, 4, 2, 64, 16, 300),     # 16 chunks, uint16 right index
+                                                 (2, 200, 14336, 3, 4, 128, 16, 256),   # 7 chunks per wave
+                                                 (1, 96, 512, 4, 4, 512, 8, 8)])        # group longer than a chunk: portable
 def test_mm_T(oracle, M, N, K, Sl, Sr, G, Ll, Lr):
     import sbvr
     dev = torch.device("cuda:0")
