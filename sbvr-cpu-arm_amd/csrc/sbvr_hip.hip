@@ -726,7 +726,10 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             const size_t at = (static_cast<size_t>(t / a.steps_per_group) * N + n_ld) << a.idx16;
             const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
             const int lo = ib[at], hi = ib[at + a.idx16];
-            return min(a.idx16 ? lo | (hi << 8) : lo, a.L - 1);
+            return lo | (hi << 16);          // raw bytes: put together where the index is used, not here,
+        };                                   // or the wait for this youngest load would drain all loads
+        auto line_of = [&](int raw) __attribute__((always_inline)) -> int {
+            return min(a.idx16 ? (raw & 0xff) | ((raw >> 8) & 0xff00) : raw & 0xff, a.L - 1);
         };
         // global loads of tile t into one register set
         auto request = [&](int t, v4u (&ar)[8], uint32_t (&wr)[S], uint32_t (&cr)[CW]) __attribute__((always_inline)) {
@@ -739,7 +742,7 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
 #pragma unroll
             for (int j = 0; j < S; ++j)
                 wr[j] = pl.w[j];
-            const uint16_t *cp = a.cache + static_cast<size_t>(line[0]) * S;
+            const uint16_t *cp = a.cache + static_cast<size_t>(line_of(line[0])) * S;
 #pragma unroll
             for (int j = 0; j < (S + 1) / 2; ++j) {
                 if (S % 2 == 0 || 2 * j + 1 < S)
@@ -943,7 +946,7 @@ sbvr_gemm_rows32_kernel(const RowsArgs a)
             const size_t at = (static_cast<size_t>(w / a.words_per_group) * N + n_ld) << a.idx16;
             const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
             const int lo = ib[at], hi = ib[at + a.idx16];      // two byte loads whatever the width: no branch
-            line[i] = min(a.idx16 ? lo | (hi << 8) : lo, a.L - 1);
+            line[i] = lo | (hi << 16);                          // raw: decoded where it is used (see the prefill kernel)
         }
     };
     auto load_block = [&](int w0, Block &b, const int (&line)[kRowsBlock]) __attribute__((always_inline)) {
@@ -965,7 +968,8 @@ sbvr_gemm_rows32_kernel(const RowsArgs a)
                 b.xa[i][0] = *reinterpret_cast<const v4u *>(xrow + 32 * w);
                 b.xa[i][1] = *reinterpret_cast<const v4u *>(xrow + 32 * w + 16);
             }
-            const uint16_t *cp = a.cache + static_cast<size_t>(line[i]) * S;
+            const int ln = min(a.idx16 ? (line[i] & 0xff) | ((line[i] >> 8) & 0xff00) : line[i] & 0xff, a.L - 1);
+            const uint16_t *cp = a.cache + static_cast<size_t>(ln) * S;
 #pragma unroll
             for (int q = 0; q < CW; ++q) {
                 if (S % 2 == 0 || 2 * q + 1 < S)
@@ -1104,7 +1108,11 @@ hipError_t launch_gemm(int S, const GemmArgs &a, hipStream_t st)
     const size_t lds = 2 * (kGemmATile + kGemmBTile);      // 96 KiB: above the 64 KiB a kernel gets without asking
 #define SBVR_GEMM_LAUNCH(SS)                                                                                   \
     {                                                                                                          \
-        static bool raised = false;                                                                            \
+        static bool raised_on[16] = {};                                                                        \
+        int dev_now = 0;                                                                                       \
+        if (hipGetDevice(&dev_now) != hipSuccess || dev_now < 0 || dev_now >= 16)                              \
+            dev_now = 0;                                                                                       \
+        bool &raised = raised_on[dev_now];                                                                     \
         if (!raised) {                                                                                         \
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sbvr_gemm_mfma_kernel<SS>), \
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
@@ -1245,7 +1253,7 @@ sbvr_mm_T_popc_kernel(const uint32_t *__restrict__ l_bvr, const uint8_t *__restr
             // one line index per group; read per word (same address within a group: cached)
             const size_t at = (static_cast<size_t>(w / wpg) * N + n_ld) << r_idx16;
             const int lo = r_idx[at], hi = r_idx[at + r_idx16];
-            line[i] = min(r_idx16 ? lo | (hi << 8) : lo, Lr - 1);
+            line[i] = lo | (hi << 16);                              // raw: decoded where it is used
         }
     };
 
@@ -1277,7 +1285,8 @@ sbvr_mm_T_popc_kernel(const uint32_t *__restrict__ l_bvr, const uint8_t *__restr
                 const int llo = l_idx[lat], lhi = l_idx[lat + l_idx16];
                 const int lline = __builtin_amdgcn_readfirstlane(min(l_idx16 ? llo | (lhi << 8) : llo, Ll - 1));
                 const uint16_t *ca = l_cache + static_cast<size_t>(lline) * SL;
-                const uint16_t *cb = r_cache + static_cast<size_t>(line[i]) * SR;
+                const int rline = min(r_idx16 ? (line[i] & 0xff) | ((line[i] >> 8) & 0xff00) : line[i] & 0xff, Lr - 1);
+                const uint16_t *cb = r_cache + static_cast<size_t>(rline) * SR;
                 float group = 0.f;
 #pragma unroll
                 for (int r = 0; r < SR; ++r) {
