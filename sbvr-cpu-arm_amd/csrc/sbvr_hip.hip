@@ -647,23 +647,25 @@ hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t 
 // ------------------------------------------------------------- MFMA prefill
 
 // Prefill path (M > 16): a dense contraction.  A workgroup owns a 256 x 128
-// tile of the output and walks K in steps of 64.  Its 8 waves have two jobs:
-//   * waves 4-7 produce the LDS tiles of step t+1 while step t is consumed:
-//     they copy the 256 x 64 activations as they are and decode the 128 x 64
-//     weights to fp16: thread (column, word) holds the S plane words of one
-//     32-bit word of K and the coefficient line of its group, and forms
-//     w = sum_j (bit_j ? c_j : 0), two elements (k, k+16) per packed fp16
-//     operation: (word >> k) & 0x00010001 times the 16-bit pattern of c_j is
-//     that pattern, or zero, in each half.  Their global loads run three steps
-//     ahead of the consumers, in three register sets used in rotation;
+// tile of the output and walks K in steps of 64.  Its 12 waves have two jobs:
+//   * waves 4-11 produce the weight tile of step t+1 while step t is consumed:
+//     128 x 64 weights decoded to fp16: thread (column, word, half) holds the
+//     S plane words of one 32-bit word of K and the coefficient line of its
+//     group, and forms w = sum_j (bit_j ? c_j : 0) for 16 of the word's
+//     elements, two of them (k, k+16) per packed fp16 operation:
+//     (word >> k) & 0x00010001 times the 16-bit pattern of c_j is that pattern,
+//     or zero, in each half.  Their global loads run three steps ahead of the
+//     consumers, in three register sets used in rotation;
 //   * waves 0-3 run v_mfma_f32_32x32x16_f16 over the two tiles (each wave
-//     128 x 64 of the output, 8 accumulator blocks).
-// A SIMD holds one wave of each kind, so the decode (VALU) and the MFMAs
-// overlap.  Both tiles are double-buffered; one barrier per step.  Rows of the
+//     128 x 64 of the output, 8 accumulator blocks) and, before that, send for
+//     the 256 x 64 activations of the next step: global memory to LDS directly,
+//     no registers, the data lands while the MFMAs run.
+// A SIMD holds one consumer and two producers, so the decode (VALU) and the
+// MFMAs overlap.  Both tiles are double-buffered; one barrier per step.  Rows of the
 // LDS tiles are 128 bytes; 16-byte chunk c of row r is stored at chunk
 // c ^ (r & 7), which keeps the 16-byte operand reads of a quarter wave on
 // different banks.
-constexpr int kGemmBM = 256, kGemmBN = 128, kGemmBK = 64, kGemmThreads = 512;
+constexpr int kGemmBM = 256, kGemmBN = 128, kGemmBK = 64, kGemmThreads = 768;     // 4 consumer + 8 producer waves
 constexpr int kGemmATile = kGemmBM * kGemmBK * 2, kGemmBTile = kGemmBN * kGemmBK * 2;
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -681,11 +683,24 @@ struct GemmArgs {
     int M, N, K, L;
     int steps_per_group;   // G / 64
     int idx16;
+#ifdef SBVR_TRACE
+    unsigned long long *trace;
+#endif
 };
+
+#ifdef SBVR_TRACE
+#define SBVR_GSTAMP(step, slot)                                                                   \
+    do {                                                                                          \
+        if (a.trace && blockIdx.x == 7 && blockIdx.y == 1 && (threadIdx.x & 63) == 0 && (step) < 96) \
+            a.trace[(step) * 8 + (slot)] = wall_clock64();                                        \
+    } while (0)
+#else
+#define SBVR_GSTAMP(step, slot) do { } while (0)
+#endif
 
 template <int S>
 __global__ void __launch_bounds__(kGemmThreads)
-__attribute__((amdgpu_waves_per_eu(2, 2)))
+__attribute__((amdgpu_waves_per_eu(3, 3)))
 sbvr_gemm_mfma_kernel(const GemmArgs a)
 {
     extern __shared__ __align__(16) unsigned char gsm[];
@@ -702,21 +717,14 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
     if (wave >= 4) {
         // ------------------------------------------------------------ producers
         const int pt = tid - 256;
-        const int bn = pt & (kGemmBN - 1), bw = pt >> 7;  // decode role: column of the tile, word of the step
+        // decode role: column of the tile, word of the step, and which 8 of the word's 16 pairs (k, k+16)
+        const int bn = pt & (kGemmBN - 1), bw = (pt >> 7) & 1, bh = pt >> 8;
         const int n_ld = min(n0 + bn, N - 1);
-        // copy role: chunk q = pt + 256 i of the step's 2048 16-byte chunks: row q / 8, chunk q % 8
-        uint32_t xoff[8];
-        const int row0 = pt >> 3, c0 = pt & 7;
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            xoff[i] = static_cast<uint32_t>(min(m0 + row0 + 32 * i, M - 1)) * K + c0 * 8;     // M * K < 2^31 (checked)
-        const int a_dst = row0 * 128 + ((c0 ^ (row0 & 7)) << 4);       // + 4096 i
         const int b_dst = bn * 128;
         const int sw = bn & 7, cb = bw * 4;
 
         constexpr int CW = (S + 1) / 2;
-        v4u areg0[8], areg1[8], areg2[8];                // three register sets, used in rotation
-        uint32_t wreg0[S], wreg1[S], wreg2[S];
+        uint32_t wreg0[S], wreg1[S], wreg2[S];           // three register sets, used in rotation
         uint32_t creg0[CW], creg1[CW], creg2[CW];
         int line[2] = {0, 0};       // line index of the tile to be requested next, and of the one after
 
@@ -732,11 +740,8 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             return min(a.idx16 ? (raw & 0xff) | ((raw >> 8) & 0xff00) : raw & 0xff, a.L - 1);
         };
         // global loads of tile t into one register set
-        auto request = [&](int t, v4u (&ar)[8], uint32_t (&wr)[S], uint32_t (&cr)[CW]) __attribute__((always_inline)) {
+        auto request = [&](int t, uint32_t (&wr)[S], uint32_t (&cr)[CW]) __attribute__((always_inline)) {
             const int k0 = t * kGemmBK;
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                ar[i] = *reinterpret_cast<const v4u *>(a.x + xoff[i] + k0);
             const uint32_t *wp = a.bvr + (static_cast<size_t>(k0 / 32 + bw) * N + n_ld) * S;
             const Planes<S> pl = load_planes<S>(wp);
 #pragma unroll
@@ -754,41 +759,34 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             line[1] = load_line(min(t + 2, steps - 1));
         };
         // one register set -> LDS buffers t % 2
-        auto produce = [&](int t, const v4u (&ar)[8], const uint32_t (&wr)[S], const uint32_t (&cr)[CW]) __attribute__((always_inline)) {
-            unsigned char *At = As + (t & 1) * kGemmATile, *Bt = Bs + (t & 1) * kGemmBTile;
+        auto produce = [&](int t, const uint32_t (&wr)[S], const uint32_t (&cr)[CW]) __attribute__((always_inline)) {
+            unsigned char *Bt = Bs + (t & 1) * kGemmBTile;
             uint32_t cbits[S];
 #pragma unroll
             for (int j = 0; j < S; ++j)
                 cbits[j] = j & 1 ? cr[j / 2] >> 16 : cr[j / 2] & 0xffffu;
-            uint32_t pr[16];         // pr[k] = {w[k], w[k+16]}
+            uint32_t wsh[S];
 #pragma unroll
-            for (int k = 0; k < 16; ++k) {
-                v2h v = __builtin_bit_cast(v2h, __umul24((wr[0] >> k) & 0x00010001u, cbits[0]));
+            for (int j = 0; j < S; ++j)
+                wsh[j] = wr[j] >> (8 * bh);
+            uint32_t pr[8];          // pr[e] = {w[8 bh + e], w[16 + 8 bh + e]}
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v2h v = __builtin_bit_cast(v2h, __umul24((wsh[0] >> e) & 0x00010001u, cbits[0]));
 #pragma unroll
                 for (int j = 1; j < S; ++j)
-                    v = v + __builtin_bit_cast(v2h, __umul24((wr[j] >> k) & 0x00010001u, cbits[j]));
-                pr[k] = __builtin_bit_cast(uint32_t, v);
+                    v = v + __builtin_bit_cast(v2h, __umul24((wsh[j] >> e) & 0x00010001u, cbits[j]));
+                pr[e] = __builtin_bit_cast(uint32_t, v);
             }
-            v4u q[4];                // k 0..7, 8..15 (low halves), 16..23, 24..31 (high halves)
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const uint32_t sel = h ? 0x07060302u : 0x05040100u;
-#pragma unroll
-                for (int g = 0; g < 2; ++g) {
-                    q[2 * h + g].x = __builtin_amdgcn_perm(pr[8 * g + 1], pr[8 * g + 0], sel);
-                    q[2 * h + g].y = __builtin_amdgcn_perm(pr[8 * g + 3], pr[8 * g + 2], sel);
-                    q[2 * h + g].z = __builtin_amdgcn_perm(pr[8 * g + 5], pr[8 * g + 4], sel);
-                    q[2 * h + g].w = __builtin_amdgcn_perm(pr[8 * g + 7], pr[8 * g + 6], sel);
-                }
-            }
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                *reinterpret_cast<v4u *>(Bt + b_dst + (((cb + c) ^ sw) << 4)) = q[c];
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                *reinterpret_cast<v4u *>(At + a_dst + 4096 * i) = ar[i];
+            v4u lo, hi;              // k 8 bh .. + 7 (low halves) and 16 + 8 bh .. + 7 (high halves)
+            lo.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x05040100u); hi.x = __builtin_amdgcn_perm(pr[1], pr[0], 0x07060302u);
+            lo.y = __builtin_amdgcn_perm(pr[3], pr[2], 0x05040100u); hi.y = __builtin_amdgcn_perm(pr[3], pr[2], 0x07060302u);
+            lo.z = __builtin_amdgcn_perm(pr[5], pr[4], 0x05040100u); hi.z = __builtin_amdgcn_perm(pr[5], pr[4], 0x07060302u);
+            lo.w = __builtin_amdgcn_perm(pr[7], pr[6], 0x05040100u); hi.w = __builtin_amdgcn_perm(pr[7], pr[6], 0x07060302u);
+            *reinterpret_cast<v4u *>(Bt + b_dst + (((cb + bh) ^ sw) << 4)) = lo;
+            *reinterpret_cast<v4u *>(Bt + b_dst + (((cb + 2 + bh) ^ sw) << 4)) = hi;
         };
-#define SBVR_SET(n) areg##n, wreg##n, creg##n
+#define SBVR_SET(n) wreg##n, creg##n
         // Requests are never conditional (beyond the last tile they repeat it): after a
         // branch that may or may not have issued loads, the wait for an older set would
         // have to assume it had not, and wait for everything.
@@ -805,14 +803,23 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             const int i = 3 * r;
             // (tiles beyond the last are produced too, from repeated loads, into buffers nobody reads:
             // a loop body without branches keeps the waits of the three register sets apart)
+            if (wave == 4) SBVR_GSTAMP(i, 2);
             request(min(i + 3, last), SBVR_SET(0));
+            if (wave == 4) SBVR_GSTAMP(i, 3);
             produce(i + 1, SBVR_SET(1));
+            if (wave == 4) SBVR_GSTAMP(i, 4);
             __syncthreads();
+            if (wave == 4) SBVR_GSTAMP(i + 1, 2);
             request(min(i + 4, last), SBVR_SET(1));
+            if (wave == 4) SBVR_GSTAMP(i + 1, 3);
             produce(i + 2, SBVR_SET(2));
+            if (wave == 4) SBVR_GSTAMP(i + 1, 4);
             __syncthreads();
+            if (wave == 4) SBVR_GSTAMP(i + 2, 2);
             request(min(i + 5, last), SBVR_SET(2));
+            if (wave == 4) SBVR_GSTAMP(i + 2, 3);
             produce(i + 3, SBVR_SET(0));
+            if (wave == 4) SBVR_GSTAMP(i + 2, 4);
             __syncthreads();
         }
 #undef SBVR_SET
@@ -831,6 +838,25 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
     const int wm = wave >> 1, wn = wave & 1;
     const int arow = wm * 128 + (lane & 31), brow = wn * 64 + (lane & 31);      // + 32 bi / bj: same row & 7
     const int rsw = lane & 7, chi = lane >> 5;
+    // The activation tile goes from global memory straight into LDS (no registers): instruction j
+    // of wave w fills the 1 KiB block 8w + j, i.e. rows 8 (8w + j) .. + 7, lane l the 16-byte slot l
+    // of it; with the row swizzle, slot l of a block holds chunk (l & 7) ^ (l >> 3) of row l >> 3.
+    uint32_t xoff[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int row = 8 * (8 * wave + j) + (lane >> 3);
+        xoff[j] = static_cast<uint32_t>(min(m0 + row, M - 1)) * K + 8 * ((lane & 7) ^ (lane >> 3));     // M * K < 2^31 (checked)
+    }
+    auto fetch_a = [&](int t) __attribute__((always_inline)) {        // tile t -> buffer t % 2, asynchronously
+        unsigned char *dst = As + (t & 1) * kGemmATile + wave * 8192;
+        const uint16_t *src = a.x + static_cast<size_t>(t) * kGemmBK;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + xoff[j]),
+                                             (__attribute__((address_space(3))) void *)(dst + j * 1024), 16, 0, 0);
+    };
+    fetch_a(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): the tile is in LDS
     __syncthreads();
     // operand registers of two k-slices in turn: the reads of slice s+1 are issued before the MFMAs of slice s
     auto read_slice = [&](const unsigned char *At, const unsigned char *Bt, int ks, v8h (&af)[4], v8h (&bf)[2])
@@ -853,6 +879,8 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
     for (int i = 0; i < 3 * rounds; ++i) {
         if (i < steps) {
             const unsigned char *At = As + (i & 1) * kGemmATile, *Bt = Bs + (i & 1) * kGemmBTile;
+            if (wave == 0) SBVR_GSTAMP(i, 0);
+            fetch_a(min(i + 1, steps - 1));      // lands in the other buffer while this one is used
             v8h af0[4], bf0[2], af1[4], bf1[2];
             read_slice(At, Bt, 0, af0, bf0);
             read_slice(At, Bt, 1, af1, bf1);
@@ -862,6 +890,8 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             read_slice(At, Bt, 3, af1, bf1);
             mfma_slice(af0, bf0);
             mfma_slice(af1, bf1);
+            if (wave == 0) SBVR_GSTAMP(i, 1);
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the next tile is in LDS
         }
         __syncthreads();
     }
@@ -1469,6 +1499,9 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
         g.M = M; g.N = N; g.K = K; g.L = L;
         g.steps_per_group = G / kGemmBK;
         g.idx16 = idx_bytes == 2;
+#ifdef SBVR_TRACE
+        g.trace = g_trace;
+#endif
         const hipError_t e = launch_gemm(S, g, st);
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "gemm launch: %s", hipGetErrorString(e));
