@@ -303,17 +303,20 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
                     xx[sgi][mt][r] = reinterpret_cast<const uint32_t *>(
                         a.x + static_cast<size_t>(mt * 4 + r) * K + static_cast<size_t>(sg0 + sgi) * kSub)[lane];
             }
-    int qline[U];
+    // line indices: one load per sub-group, lane l takes the index of column n_base + l of the
+    // window (16*CT <= 64 columns); they are handed to the (tile, column) lanes later, in LDS
+    // permutes: every vector-memory instruction saved is tens of nanoseconds of issue time
+    int lraw[SP];
     {
-        const uint32_t lane_i = static_cast<uint32_t>(n_base + col);
+        const uint32_t lane_i = static_cast<uint32_t>(n_base + min(lane, 16 * CT - 1));
         if (a.idx16) {
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                qline[u] = static_cast<const uint16_t *>(a.idx)[static_cast<size_t>((sg0 + u / CT) >> a.gshift) * N + lane_i + (u % CT) * 16];
+            for (int sgi = 0; sgi < SP; ++sgi)
+                lraw[sgi] = static_cast<const uint16_t *>(a.idx)[static_cast<size_t>((sg0 + sgi) >> a.gshift) * N + lane_i];
         } else {
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                qline[u] = static_cast<const uint8_t *>(a.idx)[static_cast<size_t>((sg0 + u / CT) >> a.gshift) * N + lane_i + (u % CT) * 16];
+            for (int sgi = 0; sgi < SP; ++sgi)
+                lraw[sgi] = static_cast<const uint8_t *>(a.idx)[static_cast<size_t>((sg0 + sgi) >> a.gshift) * N + lane_i];
         }
     }
     Planes<S> q[U];
@@ -379,27 +382,28 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     }
     SBVR_STAMP(2);
 
-    // -- 3. coefficient lines of the units (S fp16 each)
+    // -- 3. coefficient lines (S fp16 each): lane l gathers the line of column n_base + l for each
+    //       sub-group, then the (tile, column) lanes pick theirs up with LDS permutes
     constexpr int CW = (S + 1) / 2;          // dwords per line
-    uint32_t cq[U][CW];
+    uint32_t cl[SP][CW];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const uint32_t line = static_cast<uint32_t>(min(qline[u], a.L - 1));
+    for (int sgi = 0; sgi < SP; ++sgi) {
+        const uint32_t line = static_cast<uint32_t>(min(lraw[sgi], a.L - 1));
         const uint16_t *p = a.cache + line * S;
         if constexpr (S == 4) {
             const uint2 t = *reinterpret_cast<const uint2 *>(p);
-            cq[u][0] = t.x; cq[u][1] = t.y;
+            cl[sgi][0] = t.x; cl[sgi][1] = t.y;
         } else if constexpr (S == 8) {
             const uint4 t = *reinterpret_cast<const uint4 *>(p);
-            cq[u][0] = t.x; cq[u][1] = t.y; cq[u][2] = t.z; cq[u][3] = t.w;
+            cl[sgi][0] = t.x; cl[sgi][1] = t.y; cl[sgi][2] = t.z; cl[sgi][3] = t.w;
         } else if constexpr (S % 2 == 0) {
 #pragma unroll
             for (int j = 0; j < CW; ++j)
-                cq[u][j] = reinterpret_cast<const uint32_t *>(p)[j];
+                cl[sgi][j] = reinterpret_cast<const uint32_t *>(p)[j];
         } else {
 #pragma unroll
             for (int j = 0; j < CW; ++j)
-                cq[u][j] = static_cast<uint32_t>(p[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(p[2 * j + 1]) << 16 : 0u);
+                cl[sgi][j] = static_cast<uint32_t>(p[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(p[2 * j + 1]) << 16 : 0u);
         }
     }
     SBVR_STAMP(3);
@@ -447,10 +451,15 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int sgi = u / CT, ct = u % CT;
+        // (the permutes sit here, behind the units: the gathered lines are the youngest loads)
+        uint32_t cqu[CW];
+#pragma unroll
+        for (int j = 0; j < CW; ++j)
+            cqu[j] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute((ct * 16 + col) * 4, static_cast<int>(cl[sgi][j])));
         float c[S];
 #pragma unroll
         for (int j = 0; j < S; ++j)
-            c[j] = h2f(static_cast<uint16_t>(j & 1 ? cq[u][j / 2] >> 16 : cq[u][j / 2] & 0xffffu));
+            c[j] = h2f(static_cast<uint16_t>(j & 1 ? cqu[j / 2] >> 16 : cqu[j / 2] & 0xffffu));
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             float acc = 0.f;
