@@ -81,6 +81,35 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
                         void *stream);
 
 /*
+ * The same operator for one row (M = 1) with the elementwise step that feeds
+ * it folded into its activation load, which saves a kernel launch per use in a
+ * batch-1 decode step.  Same arguments as sbvr_hip_linear_f16 unless listed;
+ * only shapes the decode kernel covers (N >= 16, K and G multiples of 128 with
+ * G/128 a power of two, S in {2,3,4,6,8}); SBVR_HIP_EUNSUPPORTED otherwise (the
+ * caller then runs the two steps separately).
+ *
+ * _swiglu: gate_up is (1, 2K) fp16 = gate | up; the row multiplied with the
+ * weight is fp16(fp16(silu(gate)) * up), the argument of down_proj in
+ * models/sbvr_llama.py:238-239 (LlamaMLP.forward).
+ *
+ * _add_rmsnorm: r = fp16(x + delta) is written to x_out, and the row
+ * multiplied with the weight is norm_weight * fp16(r * rsqrt(mean(r^2) + eps)):
+ * the residual add of models/sbvr_llama.py:396-400 (LlamaDecoderLayer.forward)
+ * followed by LlamaRMSNorm.forward, :118-124.  x, delta, x_out: (K) fp16,
+ * 16-byte aligned; x_out must not be x or delta.  K <= 16384.
+ */
+int sbvr_hip_linear_f16_swiglu(const void *gate_up, const uint32_t *bvr, const void *coeff_idx,
+                               int idx_bytes, const void *coeff_cache, const void *bias,
+                               void *out, int M, int N, int K, int S, int G, int L,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
+int sbvr_hip_linear_f16_add_rmsnorm(const void *x, const void *delta, const void *norm_weight, float eps,
+                                    void *x_out, const uint32_t *bvr, const void *coeff_idx,
+                                    int idx_bytes, const void *coeff_cache, const void *bias,
+                                    void *out, int N, int K, int S, int G, int L,
+                                    void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * fp16 activations against a weight encoded with trans=True (groups along N):
  *   r_bvr (N/32, K, S) uint32, r_coeff_idx (N/G, K), r_coeff_cache (L, S) fp16
  *   out[m,n] = f16( bias[n] + sum_k x[m,k] * sum_j c[idx[n/G,k], j] * bit_j )

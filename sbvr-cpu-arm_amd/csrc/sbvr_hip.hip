@@ -43,6 +43,7 @@ namespace {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
 thread_local char g_err[256] = "";
 
@@ -154,6 +155,12 @@ struct GemvArgs {
     int gshift;           // a coefficient group is 128 << gshift elements
     int idx16;            // line indices are uint16 (else uint8)
     int ksplit;           // workgroups along K
+    int xstride;          // elements between batch rows of x
+    // fused activation prologues (see XM of the kernel)
+    const uint16_t *delta;      // XM == 2: added to x before the norm
+    const uint16_t *norm_w;     // XM == 2: RMSNorm weight
+    uint16_t *x_out;            // XM == 2: receives fp16(x + delta)
+    float eps;
 #ifdef SBVR_TRACE
     unsigned long long *trace;   // 8 timestamps per workgroup (development builds only)
 #endif
@@ -240,6 +247,58 @@ __device__ __forceinline__ uint32_t wave_umax(uint32_t v)
     return max(max(r0, r1), max(r2, r3));
 }
 
+// sum over the 64 lanes; the result is wave-uniform
+__device__ __forceinline__ float wave_fsum(float v)
+{
+#define SBVR_DPP_ADD(ctrl) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xF, 0xF, true))
+    SBVR_DPP_ADD(0xB1);      // quad_perm 1,0,3,2
+    SBVR_DPP_ADD(0x4E);      // quad_perm 2,3,0,1
+    SBVR_DPP_ADD(0x141);     // row_half_mirror
+    SBVR_DPP_ADD(0x140);     // row_mirror
+#undef SBVR_DPP_ADD
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// Activation prologues of the decode kernel: what the A operands are made from.
+//   kXPlain   x itself;
+//   kXSwiGLU  M == 1, x is (1, 2K) = gate | up: fp16(fp16(silu(gate)) * up), the MLP's
+//             act_fn(gate_proj(x)) * up_proj(x) (models/sbvr_llama.py:238-239);
+//   kXAddNorm M == 1: r = fp16(x + delta), weight * fp16(r * rsqrt(mean(r^2) + eps)),
+//             the decoder layer's residual add followed by its RMSNorm
+//             (models/sbvr_llama.py:396-400 and :118-124); every workgroup works out
+//             the mean over all of K by itself, workgroup (0, 0) writes r to x_out.
+constexpr int kXPlain = 0, kXSwiGLU = 1, kXAddNorm = 2;
+constexpr int kNormChunksPerThread = 2;       // 16-byte chunks of x a thread sums for the norm
+
+__device__ __forceinline__ uint32_t swiglu_pair(uint32_t g, uint32_t u)
+{
+    auto one = [](uint16_t gh, uint16_t uh) __attribute__((always_inline)) -> uint32_t {
+        const float gf = h2f(gh);
+        const float act = h2f(f2h(gf / (1.f + __expf(-gf))));
+        return f2h(act * h2f(uh));
+    };
+    return one(static_cast<uint16_t>(g & 0xffffu), static_cast<uint16_t>(u & 0xffffu)) |
+           (one(static_cast<uint16_t>(g >> 16), static_cast<uint16_t>(u >> 16)) << 16);
+}
+
+__device__ __forceinline__ uint32_t add_pair(uint32_t x, uint32_t d)
+{
+    const uint32_t lo = f2h(h2f(static_cast<uint16_t>(x & 0xffffu)) + h2f(static_cast<uint16_t>(d & 0xffffu)));
+    const uint32_t hi = f2h(h2f(static_cast<uint16_t>(x >> 16)) + h2f(static_cast<uint16_t>(d >> 16)));
+    return lo | (hi << 16);
+}
+
+__device__ __forceinline__ uint32_t norm_pair(uint32_t r, uint32_t w, float inv)
+{
+    const uint32_t lo = f2h(h2f(static_cast<uint16_t>(w & 0xffffu)) * h2f(f2h(h2f(static_cast<uint16_t>(r & 0xffffu)) * inv)));
+    const uint32_t hi = f2h(h2f(static_cast<uint16_t>(w >> 16)) * h2f(f2h(h2f(static_cast<uint16_t>(r >> 16)) * inv)));
+    return lo | (hi << 16);
+}
+
 // float -> the split-K accumulator's fixed point (2^-kAccFracBits), |v| <= kAccClamp.
 // hi = rint(y * 2^(F-24)) and lo = y * 2^F - hi * 2^24 are exact in fp32.
 __device__ __forceinline__ long long to_fixed(float y)
@@ -266,7 +325,7 @@ __device__ __forceinline__ long long to_fixed(float y)
 //   4. every unit: four ANDs per plane word, MFMA, plane sums kept in registers;
 //   5. coefficients applied; partial results to LDS, barrier, summed in a fixed
 //      order by the first waves, written out (or added to the split-K words).
-template <int S, int MT, int CT, int SP>
+template <int S, int MT, int CT, int SP, int XM>
 __global__ void __launch_bounds__(64 * kMaxWaves)
 __attribute__((amdgpu_waves_per_eu(gemv_waves(S, MT, CT, SP), 8)))
 sbvr_gemv_mfma_kernel(const GemvArgs a)
@@ -292,6 +351,9 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     // -- 1. requests.  Unit u = (sub-group u / CT, column tile u % CT).
     constexpr int U = SP * CT;
     uint32_t xx[SP][MT][4];
+    uint32_t x2[XM == kXPlain ? 1 : SP][XM == kXPlain ? 1 : MT][4];     // up (SwiGLU), delta (add + norm)
+    uint32_t xw[XM == kXAddNorm ? SP : 1];                              // norm weights
+    v4u sx[kNormChunksPerThread], sd[kNormChunksPerThread];             // this thread's share of all of x and delta
 #pragma unroll
     for (int sgi = 0; sgi < SP; ++sgi)
 #pragma unroll
@@ -299,10 +361,29 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 xx[sgi][mt][r] = 0u;
-                if (mt * 4 + r < a.M)      // wave-uniform
-                    xx[sgi][mt][r] = reinterpret_cast<const uint32_t *>(
-                        a.x + static_cast<size_t>(mt * 4 + r) * K + static_cast<size_t>(sg0 + sgi) * kSub)[lane];
+                if constexpr (XM != kXPlain)
+                    x2[sgi][mt][r] = 0u;
+                if (XM != kXPlain ? mt * 4 + r < 1 : mt * 4 + r < a.M) {    // wave-uniform; one row with a prologue
+                    const size_t at = static_cast<size_t>(mt * 4 + r) * a.xstride + static_cast<size_t>(sg0 + sgi) * kSub;
+                    xx[sgi][mt][r] = reinterpret_cast<const uint32_t *>(a.x + at)[lane];
+                    if constexpr (XM == kXSwiGLU)
+                        x2[sgi][mt][r] = reinterpret_cast<const uint32_t *>(a.x + at + K)[lane];
+                    if constexpr (XM == kXAddNorm)
+                        x2[sgi][mt][r] = reinterpret_cast<const uint32_t *>(a.delta + at)[lane];
+                }
             }
+    if constexpr (XM == kXAddNorm) {
+#pragma unroll
+        for (int sgi = 0; sgi < SP; ++sgi)
+            xw[sgi] = reinterpret_cast<const uint32_t *>(a.norm_w + static_cast<size_t>(sg0 + sgi) * kSub)[lane];
+        // (never conditional: a chunk past the end repeats the last one and is left out of the sum)
+#pragma unroll
+        for (int j = 0; j < kNormChunksPerThread; ++j) {
+            const int c = min(tid + j * static_cast<int>(blockDim.x), (K >> 3) - 1);
+            sx[j] = reinterpret_cast<const v4u *>(a.x)[c];
+            sd[j] = reinterpret_cast<const v4u *>(a.delta)[c];
+        }
+    }
     // line indices: one load per sub-group, lane l takes the index of column n_base + l of the
     // window (16*CT <= 64 columns); they are handed to the (tile, column) lanes later, in LDS
     // permutes: every vector-memory instruction saved is tens of nanoseconds of issue time
@@ -328,6 +409,7 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
             q[u] = load_planes<S>(wrow + lane_w + (u % CT) * 16 * S);
         }
     }
+    __builtin_amdgcn_sched_barrier(0);       // every request is out before anything waits
     SBVR_STAMP(1);
 
     // -- 2. A operands.  Lane l turns elements 2l and 2l+1 of a batch row into
@@ -335,8 +417,33 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     //       lane then reads its 32 bytes back.  Row tiles go from the last one,
     //       the only one that may have fewer than 4 rows, to the first, so a row
     //       of the buffer that is not rewritten holds zeros.
+    float inv = 0.f;             // XM == kXAddNorm: rsqrt(mean((x + delta)^2) + eps)
+    if constexpr (XM == kXAddNorm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < kNormChunksPerThread; ++j) {
+            const bool counts = tid + j * static_cast<int>(blockDim.x) < (K >> 3);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t r = add_pair(sx[j][e], sd[j][e]);
+                sx[j][e] = r;
+                const float lo = h2f(static_cast<uint16_t>(r & 0xffffu)), hi = h2f(static_cast<uint16_t>(r >> 16));
+                ss += counts ? fmaf(lo, lo, hi * hi) : 0.f;
+            }
+        }
+        ss = wave_fsum(ss);
+        float *const sums = reinterpret_cast<float *>(smem + waves * 2048);
+        if (lane == 0)
+            sums[wave] = ss;
+        __syncthreads();
+        float total = 0.f;
+        for (int w = 0; w < waves; ++w)
+            total += sums[w];
+        inv = rsqrtf(total / static_cast<float>(K) + a.eps);
+    }
     v8i A[SP][MT];
     float scale[SP][MT];         // of this lane's batch row (blk)
+    const int m_rows = XM != kXPlain ? 1 : a.M;
     {
         const int off0 = a_image_byte_offset(2 * lane, 0), off1 = a_image_byte_offset(2 * lane + 1, 0);
         const float fac0 = (lane & 1) ? 1.f : 4.f, fac1 = (lane & 1) ? 1.f : 2.f;
@@ -349,8 +456,12 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
                 scale[sgi][mt] = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    if (mt * 4 + r < a.M) {      // wave-uniform
-                        const uint32_t v = xx[sgi][mt][r];
+                    if (mt * 4 + r < m_rows) {      // wave-uniform
+                        uint32_t v = xx[sgi][mt][r];
+                        if constexpr (XM == kXSwiGLU)
+                            v = swiglu_pair(v, x2[sgi][mt][r]);
+                        if constexpr (XM == kXAddNorm)
+                            v = norm_pair(add_pair(v, x2[sgi][mt][r]), xw[sgi], inv);
                         // 2^e puts the largest magnitude of the sub-group into [32, 64)
                         // (fp16 bits order like magnitudes; subnormals count as 2^-15)
                         const uint32_t amax = wave_umax(max(v & 0x7fffu, (v >> 16) & 0x7fffu));
@@ -512,6 +623,16 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
             r = hadd(r, a.bias[n]);
         a.out[at] = r;
     }
+    if constexpr (XM == kXAddNorm) {
+        if (blockIdx.x == 0 && blockIdx.y == 0) {
+#pragma unroll
+            for (int j = 0; j < kNormChunksPerThread; ++j) {
+                const int c = tid + j * static_cast<int>(blockDim.x);
+                if (c < (K >> 3))
+                    reinterpret_cast<v4u *>(a.x_out)[c] = sx[j];
+            }
+        }
+    }
     SBVR_STAMP(6);
 }
 
@@ -547,7 +668,7 @@ bool shape_ok_for(int MT, int CT, int SP)
 //    the accumulators) when N alone does not give that many;
 //  - the largest workgroup that keeps that, but no more than 8 waves when the
 //    waves do not all fit on the chip at once (finer placement).
-GemvPlan plan_gemv(int M, int N, int K, int S, int cus)
+GemvPlan plan_gemv(int M, int N, int K, int S, int cus, int min_waves = 1)
 {
     const int nsub = K / kSub;
     const int MT = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
@@ -570,7 +691,7 @@ GemvPlan plan_gemv(int M, int N, int K, int S, int cus)
         const long total_waves = static_cast<long>(n_wgs) * parts;
         const int max_waves = total_waves > 32L * cus ? 8 : kMaxWaves;
         for (int waves = 1; waves <= kMaxWaves; ++waves) {
-            if (parts % waves || parts / waves > kMaxKsplit || (eW > 0 && waves != eW))
+            if (parts % waves || parts / waves > kMaxKsplit || (eW > 0 && waves != eW) || waves < min_waves)
                 continue;
             const int ksplit = parts / waves;
             const int U = CT * SP;
@@ -603,21 +724,21 @@ bool mfma_path_ok(int M, int N, int K, int S, int G)
            static_cast<double>(K / 32) * N * S < 2147483648.0;
 }
 
-template <int S, int MT, int CT, int SP>
+template <int S, int MT, int CT, int SP, int XM>
 hipError_t launch_gemv_inst(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
     const dim3 grid(static_cast<unsigned>(p.n_wgs), static_cast<unsigned>(p.ksplit)), block(64 * p.waves);
-    hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP>), grid, block, p.lds, st, a);
+    hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, XM>), grid, block, p.lds, st, a);
     return hipGetLastError();
 }
 
-template <int S, int MT>
+template <int S, int MT, int XM>
 hipError_t launch_gemv_shape(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
 #define SBVR_SHAPE(ct, sp)                                  \
     if constexpr (ct * MT <= 8 && (ct * sp * MT <= 16 || MT == 1)) \
         if (p.CT == ct && p.SP == sp)                       \
-            return launch_gemv_inst<S, MT, ct, sp>(a, p, st)
+            return launch_gemv_inst<S, MT, ct, sp, XM>(a, p, st)
     SBVR_SHAPE(1, 1); SBVR_SHAPE(1, 2); SBVR_SHAPE(1, 4); SBVR_SHAPE(1, 7);
     SBVR_SHAPE(2, 1); SBVR_SHAPE(2, 2); SBVR_SHAPE(2, 4); SBVR_SHAPE(2, 7);
     SBVR_SHAPE(4, 1); SBVR_SHAPE(4, 2); SBVR_SHAPE(4, 4);
@@ -625,29 +746,34 @@ hipError_t launch_gemv_shape(const GemvArgs &a, const GemvPlan &p, hipStream_t s
     return hipErrorInvalidConfiguration;
 }
 
+// (the fused prologues exist for one batch row only)
 template <int S>
-hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
+hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, int xm, hipStream_t st)
 {
+    if (xm == kXSwiGLU)
+        return p.MT == 1 ? launch_gemv_shape<S, 1, kXSwiGLU>(a, p, st) : hipErrorInvalidConfiguration;
+    if (xm == kXAddNorm)
+        return p.MT == 1 ? launch_gemv_shape<S, 1, kXAddNorm>(a, p, st) : hipErrorInvalidConfiguration;
     switch (p.MT) {
-    case 1: return launch_gemv_shape<S, 1>(a, p, st);
+    case 1: return launch_gemv_shape<S, 1, kXPlain>(a, p, st);
 #ifndef SBVR_FAST_BUILD
-    case 2: return launch_gemv_shape<S, 2>(a, p, st);
-    default: return launch_gemv_shape<S, 4>(a, p, st);
+    case 2: return launch_gemv_shape<S, 2, kXPlain>(a, p, st);
+    default: return launch_gemv_shape<S, 4, kXPlain>(a, p, st);
 #else
     default: return hipErrorInvalidConfiguration;
 #endif
     }
 }
 
-hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, hipStream_t st)
+hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, int xm, hipStream_t st)
 {
     switch (S) {
-    case 4: return launch_gemv_mt<4>(a, p, st);
+    case 4: return launch_gemv_mt<4>(a, p, xm, st);
 #ifndef SBVR_FAST_BUILD      // development builds: one plane count only
-    case 2: return launch_gemv_mt<2>(a, p, st);
-    case 3: return launch_gemv_mt<3>(a, p, st);
-    case 6: return launch_gemv_mt<6>(a, p, st);
-    case 8: return launch_gemv_mt<8>(a, p, st);
+    case 2: return launch_gemv_mt<2>(a, p, xm, st);
+    case 3: return launch_gemv_mt<3>(a, p, xm, st);
+    case 6: return launch_gemv_mt<6>(a, p, xm, st);
+    case 8: return launch_gemv_mt<8>(a, p, xm, st);
 #endif
     default: return hipErrorInvalidConfiguration;
     }
@@ -680,7 +806,6 @@ constexpr int kGemmATile = kGemmBM * kGemmBK * 2, kGemmBTile = kGemmBN * kGemmBK
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
 struct GemmArgs {
     const uint16_t *x;
@@ -1425,11 +1550,23 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G)
     return static_cast<size_t>(M) * N * sizeof(unsigned long long);
 }
 
-int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_idx,
-                        int idx_bytes, const void *coeff_cache, const void *bias,
-                        void *out, int M, int N, int K, int S, int G, int L,
-                        void *workspace, size_t workspace_bytes, int flags,
-                        void *stream)
+}  // extern "C"
+
+namespace {
+
+// What the decode kernel makes its A operands from (kXPlain: x as it is).
+struct Prologue {
+    int mode;
+    const void *delta, *norm_weight;
+    void *x_out;
+    float eps;
+};
+
+int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
+                int idx_bytes, const void *coeff_cache, const void *bias,
+                void *out, int M, int N, int K, int S, int G, int L,
+                void *workspace, size_t workspace_bytes, int flags,
+                void *stream, const Prologue &pro)
 {
     if (!x || !bvr || !coeff_idx || !coeff_cache || !out)
         return fail(SBVR_HIP_EINVAL, "null pointer argument");
@@ -1447,7 +1584,21 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
 
     const bool aligned = reinterpret_cast<uintptr_t>(bvr) % 16 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&
                          reinterpret_cast<uintptr_t>(coeff_cache) % 16 == 0;
-    if (!(flags & 3) && aligned && rows32_preferred(M, N, K, S, G, current_cus()) && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+    if (pro.mode != kXPlain) {
+        // the fused prologues live in the decode kernel only
+        if (!aligned || !mfma_path_ok(M, N, K, S, G) || M != 1)
+            return fail(SBVR_HIP_EUNSUPPORTED, "fused prologue needs M = 1 and the decode kernel's shapes (M=%d N=%d K=%d S=%d G=%d)", M, N, K, S, G);
+        if (pro.mode == kXAddNorm) {
+            if (!pro.delta || !pro.norm_weight || !pro.x_out)
+                return fail(SBVR_HIP_EINVAL, "null pointer argument");
+            if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(pro.delta) | reinterpret_cast<uintptr_t>(pro.x_out)) % 16 ||
+                reinterpret_cast<uintptr_t>(pro.norm_weight) % 4)
+                return fail(SBVR_HIP_EINVAL, "x, delta and x_out must be 16-byte aligned, norm_weight 4-byte");
+            if (pro.x_out == x || pro.x_out == pro.delta)
+                return fail(SBVR_HIP_EINVAL, "x_out must not alias x or delta (other workgroups still read them)");
+        }
+    }
+    if (pro.mode == kXPlain && !(flags & 3) && aligned && rows32_preferred(M, N, K, S, G, current_cus()) && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
         RowsArgs r{};
         r.x = static_cast<const uint16_t *>(x);
         r.bvr = bvr;
@@ -1463,8 +1614,14 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
             return fail(SBVR_HIP_ELAUNCH, "rows32 launch: %s", hipGetErrorString(e));
         return SBVR_HIP_OK;
     }
-    if (!(flags & 1) && aligned && mfma_path_ok(M, N, K, S, G)) {
-        const GemvPlan p = plan_gemv(M, N, K, S, current_cus());
+    if ((!(flags & 1) || pro.mode != kXPlain) && aligned && mfma_path_ok(M, N, K, S, G)) {
+        // add + norm: the workgroup's threads share out all of K, kNormChunksPerThread chunks of 8 each
+        const int min_waves = pro.mode == kXAddNorm ? (K / 8 + 64 * kNormChunksPerThread - 1) / (64 * kNormChunksPerThread) : 1;
+        GemvPlan p = plan_gemv(M, N, K, S, current_cus(), min_waves);
+        if (p.CT == 0 && pro.mode != kXPlain)
+            return fail(SBVR_HIP_EUNSUPPORTED, "no launch shape for the fused prologue (K=%d)", K);
+        if (pro.mode == kXAddNorm)
+            p.lds += 64;          // one partial sum of squares per wave
         if (p.CT > 0) {
         if (env_int("SBVR_HIP_SHOW_PLAN", 0))
             fprintf(stderr, "sbvr_hip plan M=%d N=%d K=%d S=%d: CT=%d SP=%d MT=%d waves=%d wgs=%d ksplit=%d\n", M, N, K, S, p.CT, p.SP, p.MT, p.waves, p.n_wgs, p.ksplit);
@@ -1479,6 +1636,11 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
         a.gshift = __builtin_ctz(static_cast<unsigned>(G / kSub));
         a.idx16 = idx_bytes == 2;
         a.ksplit = p.ksplit;
+        a.xstride = pro.mode == kXSwiGLU ? 2 * K : K;
+        a.delta = static_cast<const uint16_t *>(pro.delta);
+        a.norm_w = static_cast<const uint16_t *>(pro.norm_weight);
+        a.x_out = static_cast<uint16_t *>(pro.x_out);
+        a.eps = pro.eps;
 #ifdef SBVR_TRACE
         a.trace = g_trace;
 #endif
@@ -1490,7 +1652,7 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
                 return fail(SBVR_HIP_EINVAL, "workspace must be 8-byte aligned");
             a.acc = static_cast<unsigned long long *>(workspace);
         }
-        const hipError_t e = launch_gemv(S, a, p, st);
+        const hipError_t e = launch_gemv(S, a, p, pro.mode, st);
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "gemv launch (CT=%d SP=%d MT=%d waves=%d ksplit=%d): %s", p.CT, p.SP, p.MT, p.waves, p.ksplit, hipGetErrorString(e));
         return SBVR_HIP_OK;
@@ -1531,6 +1693,39 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
     if (e != hipSuccess)
         return fail(SBVR_HIP_ELAUNCH, "portable launch: %s", hipGetErrorString(e));
     return SBVR_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_idx,
+                        int idx_bytes, const void *coeff_cache, const void *bias,
+                        void *out, int M, int N, int K, int S, int G, int L,
+                        void *workspace, size_t workspace_bytes, int flags,
+                        void *stream)
+{
+    return linear_core(x, bvr, coeff_idx, idx_bytes, coeff_cache, bias, out, M, N, K, S, G, L, workspace,
+                       workspace_bytes, flags, stream, Prologue{kXPlain, nullptr, nullptr, nullptr, 0.f});
+}
+
+int sbvr_hip_linear_f16_swiglu(const void *gate_up, const uint32_t *bvr, const void *coeff_idx,
+                               int idx_bytes, const void *coeff_cache, const void *bias,
+                               void *out, int M, int N, int K, int S, int G, int L,
+                               void *workspace, size_t workspace_bytes, void *stream)
+{
+    return linear_core(gate_up, bvr, coeff_idx, idx_bytes, coeff_cache, bias, out, M, N, K, S, G, L, workspace,
+                       workspace_bytes, 0, stream, Prologue{kXSwiGLU, nullptr, nullptr, nullptr, 0.f});
+}
+
+int sbvr_hip_linear_f16_add_rmsnorm(const void *x, const void *delta, const void *norm_weight, float eps,
+                                    void *x_out, const uint32_t *bvr, const void *coeff_idx,
+                                    int idx_bytes, const void *coeff_cache, const void *bias,
+                                    void *out, int N, int K, int S, int G, int L,
+                                    void *workspace, size_t workspace_bytes, void *stream)
+{
+    return linear_core(x, bvr, coeff_idx, idx_bytes, coeff_cache, bias, out, 1, N, K, S, G, L, workspace,
+                       workspace_bytes, 0, stream, Prologue{kXAddNorm, delta, norm_weight, x_out, eps});
 }
 
 int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_coeff_idx,

@@ -8,10 +8,11 @@ import torch
 
 from .core import sbvr, _sbvr_serialized, load, mm_T
 from .hip import (_sbvr_hip_init, _sbvr_cuda_init, _sbvr_mm_T, _sbvr_row_deq_mm_T,
-                  _sbvr_linear_f16, SbvrHipError)
+                  _sbvr_linear_f16, _sbvr_linear_f16_swiglu, _sbvr_linear_f16_add_rmsnorm, SbvrHipError)
 from .linear import SBVRLinear
 
 torch.serialization.add_safe_globals([_sbvr_serialized])
 
 __all__ = ["sbvr", "_sbvr_serialized", "load", "mm_T", "_sbvr_hip_init", "_sbvr_cuda_init",
-           "_sbvr_mm_T", "_sbvr_row_deq_mm_T", "_sbvr_linear_f16", "SBVRLinear", "SbvrHipError"]
+           "_sbvr_mm_T", "_sbvr_row_deq_mm_T", "_sbvr_linear_f16", "_sbvr_linear_f16_swiglu",
+           "_sbvr_linear_f16_add_rmsnorm", "SBVRLinear", "SbvrHipError"]

@@ -59,10 +59,23 @@ class _Linear:
     def __call__(self, x):
         return hip._sbvr_linear_f16(x, self.bvr, self.idx, self.cache, None, self.bvr_len, out=self.out)
 
+    def after_swiglu(self, gate_up):
+        """The linear of silu(gate) * up, for gate_up = gate | up."""
+        return hip._sbvr_linear_f16_swiglu(gate_up, self.bvr, self.idx, self.cache, None, self.bvr_len, out=self.out)
+
+    def after_add_rmsnorm(self, x, delta, weight, eps, x_out):
+        """x_out <- x + delta, then the linear of RMSNorm(x_out) * weight."""
+        return hip._sbvr_linear_f16_add_rmsnorm(x, delta, weight, eps, x_out, self.bvr, self.idx, self.cache, None,
+                                                self.bvr_len, out=self.out)
+
 
 class SbvrLlamaDecoder:
-    def __init__(self, shape=None, device="cuda:0", num_sums=4, bvr_len=128, lines=256, max_seq=256, seed=0):
+    def __init__(self, shape=None, device="cuda:0", num_sums=4, bvr_len=128, lines=256, max_seq=256, seed=0,
+                 fused=True):
         self.shape = s = shape or LlamaShape()
+        # fused: the residual add + norm and the SiLU * up run inside the linear that follows them
+        # (5 launches per layer instead of 8)
+        self.fused = fused
         self.device = dev = torch.device(device)
         self.max_seq = max_seq
         hip._sbvr_hip_init(dev)
@@ -91,6 +104,8 @@ class SbvrLlamaDecoder:
         self.cos = torch.cos(ang).to(torch.float32).to(dev)       # (max_seq, head_dim/2)
         self.sin = torch.sin(ang).to(torch.float32).to(dev)
         self.x = torch.empty((1, s.hidden), dtype=torch.float16, device=dev)      # residual stream
+        self.x_alt = torch.empty((1, s.hidden), dtype=torch.float16, device=dev)  # its other buffer (fused steps)
+        self.zero = torch.zeros((1, s.hidden), dtype=torch.float16, device=dev)   # the first layer's "delta"
         self.h = torch.empty((1, s.hidden), dtype=torch.float16, device=dev)      # normed input of a linear
         self.ctx = torch.empty((1, q_out), dtype=torch.float16, device=dev)
         self.act = torch.empty((1, s.ffn), dtype=torch.float16, device=dev)
@@ -110,8 +125,12 @@ class SbvrLlamaDecoder:
 
     # -- one token -------------------------------------------------------------
     def step(self):
-        """One decode step: 8 launches per layer (norm, q|k|v, attention, o, norm,
-        gate|up, SiLU*up, down), the residual adds folded into the norms."""
+        """One decode step."""
+        return self._step_fused() if self.fused else self._step_unfused()
+
+    def _step_unfused(self):
+        """8 launches per layer (norm, q|k|v, attention, o, norm, gate|up,
+        SiLU*up, down), the residual adds folded into the norms."""
         s = self.shape
         x, h, ctx, act = self.x, self.h, self.ctx, self.act
         torch.index_select(self.embed, 0, self.tok, out=x)            # (1, hidden)
@@ -127,6 +146,27 @@ class SbvrLlamaDecoder:
             delta = layer["down"](act)
         hip.dec_add_rmsnorm(x, delta, self.final_norm, h, s.rms_eps)
         logits = torch.matmul(h, self.lm_head.t())                      # (1, vocab)
+        hip.dec_argmax_advance(logits, self.tok, self.generated, self.pos)
+        return logits
+
+    def _step_fused(self):
+        """5 launches per layer: q|k|v (with the residual add and norm in front),
+        attention, o, gate|up (same), down (with SiLU*up in front).  The residual
+        stream alternates between two buffers: a linear reads one and writes the
+        sum to the other, since its workgroups do not run in step."""
+        s = self.shape
+        a, b, ctx = self.x, self.x_alt, self.ctx
+        torch.index_select(self.embed, 0, self.tok, out=a)            # (1, hidden)
+        delta = self.zero
+        for layer in self.layers:
+            qkv = layer["qkv"].after_add_rmsnorm(a, delta, layer["norm1"], s.rms_eps, b)
+            hip.dec_attention(qkv, self.cos, self.sin, self.pos, layer["k"], layer["v"], ctx,
+                              s.heads, s.kv_heads, s.head_dim)
+            delta = layer["o"](ctx)
+            gate_up = layer["gate_up"].after_add_rmsnorm(b, delta, layer["norm2"], s.rms_eps, a)
+            delta = layer["down"].after_swiglu(gate_up)
+        hip.dec_add_rmsnorm(a, delta, self.final_norm, self.h, s.rms_eps)
+        logits = torch.matmul(self.h, self.lm_head.t())                 # (1, vocab)
         hip.dec_argmax_advance(logits, self.tok, self.generated, self.pos)
         return logits
 

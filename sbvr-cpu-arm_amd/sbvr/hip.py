@@ -46,6 +46,9 @@ def _load():
     lib.sbvr_hip_linear_f16_workspace.restype = sz
     lib.sbvr_hip_linear_f16_workspace.argtypes = [i, i, i, i, i]
     lib.sbvr_hip_linear_f16.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp, sz, i, vp]
+    lib.sbvr_hip_linear_f16_swiglu.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
+    lib.sbvr_hip_linear_f16_add_rmsnorm.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, vp, i, vp, vp, vp,
+                                                    i, i, i, i, i, vp, sz, vp]
     lib.sbvr_hip_row_deq_mm_T.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp]
     lib.sbvr_hip_mm_T.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
     fp = ctypes.POINTER(ctypes.c_float)
@@ -118,17 +121,13 @@ def _workspace(nbytes, device):
     return ws
 
 
-def _sbvr_linear_f16(x, bvr, coeff_idx, coeff_cache, bias=None, bvr_len=None, out=None, flags=0):
-    """y = x @ decode(W)^T (+ bias) for fp16 ``x`` (M, K) and a weight in the
-    default uint32 layout: ``bvr`` (K/32, N, S), ``coeff_idx`` (K/G, N),
-    ``coeff_cache`` (L, S).  Returns fp16 (M, N)."""
+def _linear_operands(K, bvr, coeff_idx, coeff_cache, bvr_len, out, M, dev):
+    """Shape and dtype checks shared by the linear's entry points; returns
+    (N, S, G, L, idx_bytes, out, workspace)."""
     lib = _load()
-    dev = x.device
-    _want(x, "x", torch.float16, 2)
     _want(bvr, "bvr", torch.uint32, 3, dev)
     _want(coeff_idx, "coeff_idx", (torch.uint8, torch.uint16), 2, dev)
     _want(coeff_cache, "coeff_cache", torch.float16, 2, dev)
-    M, K = x.shape
     Kw, N, S = bvr.shape
     L = coeff_cache.shape[0]
     if Kw * 32 != K:
@@ -147,12 +146,67 @@ def _sbvr_linear_f16(x, bvr, coeff_idx, coeff_cache, bias=None, bvr_len=None, ou
             raise ValueError("out has the wrong shape")
     need = lib.sbvr_hip_linear_f16_workspace(M, N, K, S, G)
     ws = _workspace(need, dev) if need else None
+    return N, S, G, L, ib, out, ws
+
+
+def _sbvr_linear_f16(x, bvr, coeff_idx, coeff_cache, bias=None, bvr_len=None, out=None, flags=0):
+    """y = x @ decode(W)^T (+ bias) for fp16 ``x`` (M, K) and a weight in the
+    default uint32 layout: ``bvr`` (K/32, N, S), ``coeff_idx`` (K/G, N),
+    ``coeff_cache`` (L, S).  Returns fp16 (M, N)."""
+    lib = _load()
+    dev = x.device
+    _want(x, "x", torch.float16, 2)
+    M, K = x.shape
+    N, S, G, L, ib, out, ws = _linear_operands(K, bvr, coeff_idx, coeff_cache, bvr_len, out, M, dev)
     with torch.cuda.device(dev):
         _check(lib.sbvr_hip_linear_f16(
             x.data_ptr(), bvr.data_ptr(), coeff_idx.data_ptr(), ib, coeff_cache.data_ptr(),
             _bias_ptr(bias, N, dev), out.data_ptr(), M, N, K, S, G, L,
             ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
             int(flags), _stream()))
+    return out
+
+
+def _sbvr_linear_f16_swiglu(gate_up, bvr, coeff_idx, coeff_cache, bias=None, bvr_len=None, out=None):
+    """``_sbvr_linear_f16`` of the row fp16(fp16(silu(gate)) * up) for ``gate_up``
+    (1, 2K) = gate | up, without materialising that row (one launch)."""
+    lib = _load()
+    dev = gate_up.device
+    _want(gate_up, "gate_up", torch.float16, 2)
+    M, K2 = gate_up.shape
+    if K2 % 2:
+        raise ValueError("gate_up must have an even number of columns")
+    K = K2 // 2
+    N, S, G, L, ib, out, ws = _linear_operands(K, bvr, coeff_idx, coeff_cache, bvr_len, out, M, dev)
+    with torch.cuda.device(dev):
+        _check(lib.sbvr_hip_linear_f16_swiglu(
+            gate_up.data_ptr(), bvr.data_ptr(), coeff_idx.data_ptr(), ib, coeff_cache.data_ptr(),
+            _bias_ptr(bias, N, dev), out.data_ptr(), M, N, K, S, G, L,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream()))
+    return out
+
+
+def _sbvr_linear_f16_add_rmsnorm(x, delta, norm_weight, eps, x_out, bvr, coeff_idx, coeff_cache, bias=None,
+                                 bvr_len=None, out=None):
+    """``x_out`` <- r = fp16(x + delta); returns ``_sbvr_linear_f16`` of the row
+    norm_weight * fp16(r * rsqrt(mean(r^2) + eps)), in one launch.  ``x``,
+    ``delta``, ``x_out``: (1, K) fp16, three different buffers."""
+    lib = _load()
+    dev = x.device
+    _want(x, "x", torch.float16, 2)
+    _want(delta, "delta", torch.float16, 2, dev)
+    _want(x_out, "x_out", torch.float16, 2, dev)
+    _want(norm_weight, "norm_weight", torch.float16, 1, dev)
+    M, K = x.shape
+    if M != 1 or tuple(delta.shape) != (1, K) or tuple(x_out.shape) != (1, K) or norm_weight.shape[0] != K:
+        raise ValueError("x, delta and x_out must be (1, K) and norm_weight (K)")
+    N, S, G, L, ib, out, ws = _linear_operands(K, bvr, coeff_idx, coeff_cache, bvr_len, out, 1, dev)
+    with torch.cuda.device(dev):
+        _check(lib.sbvr_hip_linear_f16_add_rmsnorm(
+            x.data_ptr(), delta.data_ptr(), norm_weight.data_ptr(), float(eps), x_out.data_ptr(),
+            bvr.data_ptr(), coeff_idx.data_ptr(), ib, coeff_cache.data_ptr(),
+            _bias_ptr(bias, N, dev), out.data_ptr(), N, K, S, G, L,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream()))
     return out
 
 

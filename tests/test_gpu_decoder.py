@@ -58,13 +58,14 @@ def dense_reference(dec, oracle, tokens):
     return np.stack(out)
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("graph", [False, True])
-def test_small_decoder_matches_dense(oracle, graph):
+def test_small_decoder_matches_dense(oracle, graph, fused):
     import torch
     from sbvr.decoder import LlamaShape, SbvrLlamaDecoder
 
     shape = LlamaShape(hidden=256, layers=2, heads=4, kv_heads=2, head_dim=64, ffn=512, vocab=1000)
-    dec = SbvrLlamaDecoder(shape, "cuda:0", num_sums=4, bvr_len=128, lines=64, max_seq=32, seed=5)
+    dec = SbvrLlamaDecoder(shape, "cuda:0", num_sums=4, bvr_len=128, lines=64, max_seq=32, seed=5, fused=fused)
     # weights of N(0, 0.02) leave the logits tiny; scale the tables so the layers matter
     # (not further: attention then turns one-hot and amplifies fp16 rounding into different contexts)
     for layer in dec.layers:
