@@ -29,10 +29,14 @@ int sbvr_hip_dec_add_rmsnorm_f16(void *x, const void *delta, const void *weight,
  * Replaces apply_rotary_pos_emb + the cache update + eager_attention_forward
  * (reference models/sbvr_llama.py:193-224, 255-278, 307-354) for batch 1,
  * query length 1.  *pos is read on the device, so a recorded launch can be
- * replayed for successive positions. */
-int sbvr_hip_dec_attention_f16(const void *qkv, const float *cos_table, const float *sin_table, const long long *pos,
-                               void *kcache, void *vcache, void *ctx, int heads, int kv_heads, int head_dim,
-                               int max_seq, void *stream);
+ * replayed for successive positions.  rot_now, when not NULL, holds row *pos
+ * of the two tables side by side (cos | sin, head_dim floats), as
+ * sbvr_hip_dec_argmax_advance_f16 leaves it: the kernel then need not wait
+ * for *pos before it asks for the rotation.  The caches must be 16-byte
+ * aligned. */
+int sbvr_hip_dec_attention_f16(const void *qkv, const float *cos_table, const float *sin_table, const float *rot_now,
+                               const long long *pos, void *kcache, void *vcache, void *ctx, int heads, int kv_heads,
+                               int head_dim, int max_seq, void *stream);
 
 /* out[ffn] <- fp16(silu(gate)) * up with gate_up = [gate | up] (2*ffn) fp16.
  * Replaces act_fn(gate_proj(x)) * up_proj(x) of LlamaMLP.forward
@@ -43,9 +47,13 @@ int sbvr_hip_dec_silu_mul_f16(const void *gate_up, void *out, int ffn, void *str
  * lowest index among equal maxima, as torch.argmax), generated[*pos] <- *token when
  * *pos < max_seq, *pos <- *pos + 1.  Replaces `next_tokens = argmax(logits)` and the
  * cache-position update of the generation loop the reference inherits from
- * GenerationMixin (reference models/sbvr_llama.py:801). */
+ * GenerationMixin (reference models/sbvr_llama.py:801).  When rot_now is not NULL
+ * it receives row min(*pos, max_seq - 1) (the new position) of the rotary tables
+ * cos | sin (max_seq, head_dim/2 floats each), for the attention launches of the
+ * next step. */
 int sbvr_hip_dec_argmax_advance_f16(const void *logits, int n, long long *token, long long *generated, long long *pos,
-                                    int max_seq, void *stream);
+                                    int max_seq, const float *cos_table, const float *sin_table, int head_dim,
+                                    float *rot_now, void *stream);
 
 #ifdef __cplusplus
 }

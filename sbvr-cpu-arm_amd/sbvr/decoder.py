@@ -103,6 +103,7 @@ class SbvrLlamaDecoder:
         ang = torch.arange(max_seq, dtype=torch.float64)[:, None] * inv[None, :]
         self.cos = torch.cos(ang).to(torch.float32).to(dev)       # (max_seq, head_dim/2)
         self.sin = torch.sin(ang).to(torch.float32).to(dev)
+        self.rot_now = torch.empty(s.head_dim, dtype=torch.float32, device=dev)   # cos | sin of the current position
         self.x = torch.empty((1, s.hidden), dtype=torch.float16, device=dev)      # residual stream
         self.x_alt = torch.empty((1, s.hidden), dtype=torch.float16, device=dev)  # its other buffer (fused steps)
         self.zero = torch.zeros((1, s.hidden), dtype=torch.float16, device=dev)   # the first layer's "delta"
@@ -139,14 +140,14 @@ class SbvrLlamaDecoder:
             hip.dec_add_rmsnorm(x, delta, layer["norm1"], h, s.rms_eps)
             qkv = layer["qkv"](h)
             hip.dec_attention(qkv, self.cos, self.sin, self.pos, layer["k"], layer["v"], ctx,
-                              s.heads, s.kv_heads, s.head_dim)
+                              s.heads, s.kv_heads, s.head_dim, self.rot_now)
             delta = layer["o"](ctx)
             hip.dec_add_rmsnorm(x, delta, layer["norm2"], h, s.rms_eps)
             hip.dec_silu_mul(layer["gate_up"](h), act)
             delta = layer["down"](act)
         hip.dec_add_rmsnorm(x, delta, self.final_norm, h, s.rms_eps)
         logits = torch.matmul(h, self.lm_head.t())                      # (1, vocab)
-        hip.dec_argmax_advance(logits, self.tok, self.generated, self.pos)
+        hip.dec_argmax_advance(logits, self.tok, self.generated, self.pos, self.cos, self.sin, self.rot_now)
         return logits
 
     def _step_fused(self):
@@ -161,13 +162,13 @@ class SbvrLlamaDecoder:
         for layer in self.layers:
             qkv = layer["qkv"].after_add_rmsnorm(a, delta, layer["norm1"], s.rms_eps, b)
             hip.dec_attention(qkv, self.cos, self.sin, self.pos, layer["k"], layer["v"], ctx,
-                              s.heads, s.kv_heads, s.head_dim)
+                              s.heads, s.kv_heads, s.head_dim, self.rot_now)
             delta = layer["o"](ctx)
             gate_up = layer["gate_up"].after_add_rmsnorm(b, delta, layer["norm2"], s.rms_eps, a)
             delta = layer["down"].after_swiglu(gate_up)
         hip.dec_add_rmsnorm(a, delta, self.final_norm, self.h, s.rms_eps)
         logits = torch.matmul(self.h, self.lm_head.t())                 # (1, vocab)
-        hip.dec_argmax_advance(logits, self.tok, self.generated, self.pos)
+        hip.dec_argmax_advance(logits, self.tok, self.generated, self.pos, self.cos, self.sin, self.rot_now)
         return logits
 
     # -- driving ---------------------------------------------------------------
@@ -187,6 +188,7 @@ class SbvrLlamaDecoder:
         self.pos.zero_()
         self.tok.zero_()
         self.generated.zero_()
+        self.rot_now.copy_(torch.cat((self.cos[0], self.sin[0])))
         for layer in self.layers:
             layer["k"].zero_()
             layer["v"].zero_()

@@ -53,9 +53,9 @@ def _load():
     lib.sbvr_hip_mm_T.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
     fp = ctypes.POINTER(ctypes.c_float)
     lib.sbvr_hip_dec_add_rmsnorm_f16.argtypes = [vp, vp, vp, vp, i, ctypes.c_float, vp]
-    lib.sbvr_hip_dec_attention_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
+    lib.sbvr_hip_dec_attention_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
     lib.sbvr_hip_dec_silu_mul_f16.argtypes = [vp, vp, i, vp]
-    lib.sbvr_hip_dec_argmax_advance_f16.argtypes = [vp, i, vp, vp, vp, i, vp]
+    lib.sbvr_hip_dec_argmax_advance_f16.argtypes = [vp, i, vp, vp, vp, i, vp, vp, i, vp, vp]
     _lib = lib
     return lib
 
@@ -282,8 +282,10 @@ def dec_add_rmsnorm(x, delta, weight, h, eps):
     return h
 
 
-def dec_attention(qkv, cos, sin, pos, kcache, vcache, ctx, heads, kv_heads, head_dim):
-    """Rotary embedding, cache append at *pos and attention of the new token."""
+def dec_attention(qkv, cos, sin, pos, kcache, vcache, ctx, heads, kv_heads, head_dim, rot_now=None):
+    """Rotary embedding, cache append at *pos and attention of the new token.
+    ``rot_now``: row *pos of cos | sin (head_dim floats) when the caller keeps it
+    up to date (dec_argmax_advance does), which saves the kernel a round trip."""
     for t, name in ((qkv, "qkv"), (kcache, "kcache"), (vcache, "vcache"), (ctx, "ctx")):
         _want(t, name, torch.float16)
     _want(cos, "cos", torch.float32)
@@ -294,9 +296,15 @@ def dec_attention(qkv, cos, sin, pos, kcache, vcache, ctx, heads, kv_heads, head
             cos.shape != (max_seq, head_dim // 2) or sin.shape != cos.shape or \
             qkv.numel() != (heads + 2 * kv_heads) * head_dim or ctx.numel() != heads * head_dim:
         raise SbvrHipError("dec_attention: tensor shapes do not match heads/kv_heads/head_dim/max_seq")
-    _dec_check(_load().sbvr_hip_dec_attention_f16(qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), pos.data_ptr(),
-                                                   kcache.data_ptr(), vcache.data_ptr(), ctx.data_ptr(), heads,
-                                                   kv_heads, head_dim, max_seq, _stream()), "attention")
+    if rot_now is not None:
+        _want(rot_now, "rot_now", torch.float32)
+        if rot_now.numel() != head_dim:
+            raise SbvrHipError("dec_attention: rot_now must hold head_dim floats")
+    _dec_check(_load().sbvr_hip_dec_attention_f16(qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+                                                   rot_now.data_ptr() if rot_now is not None else None,
+                                                   pos.data_ptr(), kcache.data_ptr(), vcache.data_ptr(),
+                                                   ctx.data_ptr(), heads, kv_heads, head_dim, max_seq, _stream()),
+               "attention")
     return ctx
 
 
@@ -310,11 +318,22 @@ def dec_silu_mul(gate_up, out):
     return out
 
 
-def dec_argmax_advance(logits, token, generated, pos):
-    """token <- argmax(logits); generated[pos] <- token; pos <- pos + 1 (all on the device)."""
+def dec_argmax_advance(logits, token, generated, pos, cos=None, sin=None, rot_now=None):
+    """token <- argmax(logits); generated[pos] <- token; pos <- pos + 1 (all on the device).
+    With ``rot_now`` (head_dim floats) and the rotary tables, also rot_now <- cos | sin of the new position."""
     _want(logits, "logits", torch.float16)
     for t, name in ((token, "token"), (generated, "generated"), (pos, "pos")):
         _want(t, name, torch.int64)
+    head_dim = 0
+    if rot_now is not None:
+        for t, name in ((cos, "cos"), (sin, "sin"), (rot_now, "rot_now")):
+            _want(t, name, torch.float32)
+        head_dim = rot_now.numel()
+        if cos.shape != (generated.numel(), head_dim // 2) or sin.shape != cos.shape:
+            raise SbvrHipError("dec_argmax_advance: rotary tables must be (max_seq, head_dim / 2)")
     _dec_check(_load().sbvr_hip_dec_argmax_advance_f16(logits.data_ptr(), logits.numel(), token.data_ptr(),
                                                         generated.data_ptr(), pos.data_ptr(), generated.numel(),
+                                                        cos.data_ptr() if rot_now is not None else None,
+                                                        sin.data_ptr() if rot_now is not None else None, head_dim,
+                                                        rot_now.data_ptr() if rot_now is not None else None,
                                                         _stream()), "argmax_advance")

@@ -136,3 +136,83 @@ def test_generate_is_repeatable():
     dec.graph = None
     c, _ = dec.generate(prompt, 16)
     assert torch.equal(a, c), "graph replay and eager steps disagree"
+
+
+@pytest.mark.parametrize("head_dim,max_seq,p", [(128, 256, 0), (128, 256, 5), (128, 256, 255), (128, 700, 300),
+                                                (64, 600, 511), (64, 600, 599), (64, 64, 17)])
+@pytest.mark.parametrize("ready_rotation", [False, True])
+def test_attention_kernel(head_dim, max_seq, p, ready_rotation):
+    """The attention helper by itself against numpy (fp64), with the rotation row
+    read from the tables or handed over ready, below and beyond the part of the
+    cache that the kernel requests up front (16 * 256 / (head_dim / 8) rows)."""
+    import torch
+    from sbvr import hip
+
+    dev = torch.device("cuda:0")
+    heads, kv_heads = 4, 2
+    gen = torch.Generator().manual_seed(head_dim + p)
+    qkv = torch.randn((heads + 2 * kv_heads) * head_dim, generator=gen).to(torch.float16)
+    ang = torch.rand((max_seq, head_dim // 2), generator=gen, dtype=torch.float64) * 6.28
+    cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
+    kc = torch.randn((kv_heads, max_seq, head_dim), generator=gen).to(torch.float16)
+    vc = torch.randn((kv_heads, max_seq, head_dim), generator=gen).to(torch.float16)
+    kc_d, vc_d = kc.to(dev), vc.to(dev)
+    ctx = torch.empty(heads * head_dim, dtype=torch.float16, device=dev)
+    rot = torch.cat((cos[p], sin[p])).to(dev) if ready_rotation else None
+    hip.dec_attention(qkv.to(dev), cos.to(dev), sin.to(dev), torch.tensor([p], device=dev), kc_d, vc_d, ctx,
+                      heads, kv_heads, head_dim, rot)
+    torch.cuda.synchronize()
+
+    half = head_dim // 2
+    c, s = cos[p].double().numpy(), sin[p].double().numpy()
+
+    def rope(t):
+        a, b = t[..., :half], t[..., half:]
+        return np.concatenate((a * c - b * s, b * c + a * s), axis=-1)
+
+    x = qkv.double().numpy()
+    q = rope(x[:heads * head_dim].reshape(heads, head_dim))
+    k_new = rope(x[heads * head_dim:(heads + kv_heads) * head_dim].reshape(kv_heads, head_dim))
+    v_new = x[(heads + kv_heads) * head_dim:].reshape(kv_heads, head_dim)
+    K = kc.double().numpy()[:, :p + 1].copy()
+    V = vc.double().numpy()[:, :p + 1].copy()
+    K[:, p], V[:, p] = k_new, v_new
+    want = np.zeros((heads, head_dim))
+    for h in range(heads):
+        g = h // (heads // kv_heads)
+        sc = K[g] @ q[h] / math.sqrt(head_dim)
+        pr = np.exp(sc - sc.max())
+        want[h] = (pr / pr.sum()) @ V[g]
+    got = ctx.float().cpu().numpy().astype(np.float64).reshape(heads, head_dim)
+    assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max(), np.abs(got - want).max()
+    # the caches: row p appended (rotated key, value), everything else untouched
+    kc2, vc2 = kc_d.cpu(), vc_d.cpu()
+    assert np.abs(kc2[:, p].double().numpy() - k_new).max() <= 2e-3 * np.abs(k_new).max()
+    assert torch.equal(vc2[:, p], qkv[(heads + kv_heads) * head_dim:].reshape(kv_heads, head_dim))
+    keep = torch.ones(max_seq, dtype=torch.bool)
+    keep[p] = False
+    assert torch.equal(kc2[:, keep], kc[:, keep]) and torch.equal(vc2[:, keep], vc[:, keep])
+
+
+def test_argmax_advance_leaves_rotation():
+    import torch
+    from sbvr import hip
+
+    dev = torch.device("cuda:0")
+    n, max_seq, head_dim = 1000, 8, 64
+    logits = torch.randn(n, generator=torch.Generator().manual_seed(1)).to(torch.float16)
+    logits[123] = logits[777] = 9.0                   # two equal maxima: the lower index wins
+    cos = torch.rand((max_seq, head_dim // 2)).to(dev)
+    sin = torch.rand((max_seq, head_dim // 2)).to(dev)
+    tok = torch.zeros(1, dtype=torch.int64, device=dev)
+    gen = torch.full((max_seq,), -1, dtype=torch.int64, device=dev)
+    rot = torch.zeros(head_dim, dtype=torch.float32, device=dev)
+    for start in (0, 3, 7, 8):                        # 7 -> 8 and 8 -> 9 clamp to the last row
+        pos = torch.tensor([start], dtype=torch.int64, device=dev)
+        hip.dec_argmax_advance(logits.to(dev), tok, gen, pos, cos, sin, rot)
+        torch.cuda.synchronize()
+        assert int(tok) == 123 and int(pos) == start + 1
+        if start < max_seq:
+            assert int(gen[start]) == 123
+        r = min(start + 1, max_seq - 1)
+        assert torch.equal(rot, torch.cat((cos[r], sin[r])))
