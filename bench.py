@@ -33,7 +33,7 @@ COPIES = 16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the gate GEMV, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # 256 MiB copy (profiles/sbvr_gemv_mfma_gate_4096x14336.txt): 30.43 MB read + 0.60 MB written.
-MEASURED_TRAFFIC_BYTES = 31.03e6
+MEASURED_TRAFFIC_BYTES = 31.05e6
 
 
 def algorithmic_bytes(n, k, s, g, lines, m):
