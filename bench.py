@@ -32,7 +32,7 @@ N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH = 14336, 4096, 4, 128, 256, 1
 COPIES = 16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the gate GEMV, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# 256 MiB copy (profiles/sbvr_gemv_mfma_gate_4096x14336.txt): 30.43 MB read + 0.60 MB written.
+# 256 MiB copy (profiles/sbvr_gemv_mfma_gate_4096x14336.txt): 30.45 MB read + 0.60 MB written.
 MEASURED_TRAFFIC_BYTES = 31.05e6
 
 
@@ -198,6 +198,38 @@ def sweep_leg():
     return rows
 
 
+def other_ops_leg():
+    """The reference's own operator forms at the Llama-3-8B layer shapes, batch 1: both operands
+    encoded (_sbvr_mm_T, the form its CPU kernels time) and fp16 activations against a
+    trans=True weight (_sbvr_row_deq_mm_T).  Same bytes as the linear of the same shape."""
+    import torch
+    from sbvr import synth, hip
+    dev = torch.device("cuda:0")
+    rows = []
+    none = torch.zeros(0, dtype=torch.float16, device=dev)
+    for tag, n, k in (("q/o", 4096, 4096), ("gate/up", 14336, 4096), ("down", 4096, 14336)):
+        per = n * k * NUM_SUMS // 8
+        copies = max(2, min(16, int(600e6 // per)))
+        nbytes = algorithmic_bytes(n, k, NUM_SUMS, GROUP, LINES, 1)
+        ws = [tuple(t.to(dev) for t in synth.random_encoding(n, k, NUM_SUMS, GROUP, LINES, seed=c)) for c in range(copies)]
+        left = tuple(t.to(dev) for t in synth.random_encoding(1, k, NUM_SUMS, GROUP, 16, seed=99))
+        t = _graph_time(lambda i: hip._sbvr_mm_T(*left, *ws[i % copies], none, bvr_len=GROUP), 100)
+        rows.append({"op": "_sbvr_mm_T", "linear": tag, "N": n, "K": k, "S": NUM_SUMS, "M": 1, "us": round(t * 1e6, 2),
+                     "GBps": round(nbytes / t / 1e9, 1), "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4)})
+        del ws
+        torch.cuda.empty_cache()
+        # trans=True: the encoded tensor is W^T (k rows of n columns, groups along n)
+        wt = [tuple(t.to(dev) for t in synth.random_encoding(k, n, NUM_SUMS, GROUP, LINES, seed=c)) for c in range(copies)]
+        x = torch.randn((1, k), generator=torch.Generator().manual_seed(5)).to(torch.float16).to(dev)
+        t = _graph_time(lambda i: hip._sbvr_row_deq_mm_T(x, *wt[i % copies], none, 0, bvr_len=GROUP), 100)
+        rows.append({"op": "_sbvr_row_deq_mm_T", "linear": tag, "N": n, "K": k, "S": NUM_SUMS, "M": 1,
+                     "us": round(t * 1e6, 2), "GBps": round(nbytes / t / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4)})
+        del wt
+        torch.cuda.empty_cache()
+    return rows
+
+
 def prefill_leg():
     """Prefill GEMM at the 70B-width linears, S=4, G=128: dense-equivalent TFLOP/s against
     the fp16 MFMA peak."""
@@ -299,6 +331,8 @@ def main():
     ap.add_argument("--sweep", action="store_true",
                     help="run only the layer-shape / batch / plane-count sweep of the decode kernel and print it")
     ap.add_argument("--prefill", action="store_true", help="run only the prefill GEMM sizes and print them")
+    ap.add_argument("--other-ops", action="store_true",
+                    help="run only _sbvr_mm_T and _sbvr_row_deq_mm_T at the layer shapes and print them")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size kernel that "
                          "hardware byte counters are scaled by when profiling")
@@ -314,6 +348,10 @@ def main():
         return
     if a.prefill:
         print(json.dumps({"metric": "SBVR prefill GEMM, dense-equivalent TFLOP/s", "prefill": prefill_leg()}))
+        return
+    if a.other_ops:
+        print(json.dumps({"metric": "SBVR operator forms of the reference, us and GB/s of algorithmic bytes",
+                          "other_ops": other_ops_leg()}))
         return
     if a.calibrate_copy:
         import torch

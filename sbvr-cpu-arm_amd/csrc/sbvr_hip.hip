@@ -1345,6 +1345,113 @@ sbvr_row_deq_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__
     out[o] = f2h(acc);
 }
 
+// The same product with the lanes of a wave along K.  A word of the trans=True
+// layout holds one row k of 32 columns, and rows follow each other in memory
+// (bvr[nw][k][S]), so lane l of a wave takes row 64*step + l: its plane words,
+// line index, coefficient line and activation are its own (coalesced loads, one
+// gather), z_j = x[k] * c_j is formed once, and the 32 columns of the word
+// block each get sum_j (bit_j ? z_j : 0) added to an accumulator of their own
+// (32 per lane).  A workgroup owns one block of 32 columns and one batch row;
+// its waves take the steps in turn.  At the end the 64 lanes are summed per
+// column (DPP), the waves meet in LDS and the first wave adds up, in a fixed
+// order.  The loads of a step are requested one step ahead, its line index two.
+constexpr int kRowDeqWaves = 16;
+
+template <int S>
+__global__ void __launch_bounds__(64 * kRowDeqWaves)
+sbvr_row_deq_lanes_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ bvr,
+                          const void *__restrict__ idx, const uint16_t *__restrict__ cache,
+                          const uint16_t *__restrict__ bias, uint16_t *__restrict__ out,
+                          int M, int N, int K, int L, int G, int idx16)
+{
+    __shared__ float part[kRowDeqWaves][32];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = static_cast<int>(blockDim.x >> 6);
+    const int nw = blockIdx.x, m = blockIdx.y;
+    const int steps = (K + 63) >> 6;
+    const uint32_t *wbase = bvr + static_cast<size_t>(nw) * K * S;
+    const size_t ibase = static_cast<size_t>((nw * 32) / G) * K;
+    const uint16_t *xrow = x + static_cast<size_t>(m) * K;
+
+    float acc[32];
+#pragma unroll
+    for (int b = 0; b < 32; ++b)
+        acc[b] = 0.f;
+
+    // (two byte loads whatever the index width, put together where the index is used:
+    // no branch between loads, no early wait on the youngest load)
+    auto load_line = [&](int step) __attribute__((always_inline)) -> int {
+        const size_t at = (ibase + static_cast<size_t>(min(step * 64 + lane, K - 1))) << idx16;
+        const uint8_t *ib = static_cast<const uint8_t *>(idx);
+        return static_cast<int>(ib[at]) | (static_cast<int>(ib[at + idx16]) << 16);
+    };
+    auto line_of = [&](int raw) __attribute__((always_inline)) -> int {
+        return min(idx16 ? (raw & 0xff) | ((raw >> 8) & 0xff00) : raw & 0xff, L - 1);
+    };
+    constexpr int CW = (S + 1) / 2;
+    auto load_coeffs = [&](int raw, uint32_t (&c)[CW]) __attribute__((always_inline)) {
+        const uint16_t *cp = cache + static_cast<size_t>(line_of(raw)) * S;
+#pragma unroll
+        for (int j = 0; j < CW; ++j)
+            c[j] = static_cast<uint32_t>(cp[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(cp[2 * j + 1]) << 16 : 0u);
+    };
+    const int last = steps - 1;
+    // pipeline: raw index of step i+2, and words / coefficients / activation of step i+1
+    int raw_next = load_line(min(wave, last));
+    int raw_after = load_line(min(wave + waves, last));
+    Planes<S> w_next = load_planes<S>(wbase + static_cast<size_t>(min(min(wave, last) * 64 + lane, K - 1)) * S);
+    uint16_t x_next = xrow[min(min(wave, last) * 64 + lane, K - 1)];
+    uint32_t c_next[CW];
+    load_coeffs(raw_next, c_next);
+
+    for (int step = wave; step < steps; step += waves) {
+        const Planes<S> w = w_next;
+        uint32_t c[CW];
+#pragma unroll
+        for (int j = 0; j < CW; ++j)
+            c[j] = c_next[j];
+        const float xv = step * 64 + lane < K ? h2f(x_next) : 0.f;
+        // requests of the following steps (beyond the end they repeat the last step)
+        const int s1 = min(step + waves, last), s2 = min(step + 2 * waves, last);
+        w_next = load_planes<S>(wbase + static_cast<size_t>(min(s1 * 64 + lane, K - 1)) * S);
+        x_next = xrow[min(s1 * 64 + lane, K - 1)];
+        load_coeffs(raw_after, c_next);
+        raw_after = load_line(s2);
+
+        uint32_t z[S];
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+            z[j] = __float_as_uint(xv * h2f(static_cast<uint16_t>(j & 1 ? c[j / 2] >> 16 : c[j / 2] & 0xffffu)));
+#pragma unroll
+        for (int b = 0; b < 32; ++b) {
+#pragma unroll
+            for (int j = 0; j < S; ++j) {
+                // all ones where bit b of the plane word is set
+                const uint32_t mask = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(w.w[j]), b, 1));
+                acc[b] += __uint_as_float(z[j] & mask);
+            }
+        }
+    }
+
+    float mine = 0.f;
+#pragma unroll
+    for (int b = 0; b < 32; ++b) {
+        const float v = wave_fsum(acc[b]);
+        mine = lane == b ? v : mine;
+    }
+    if (lane < 32)
+        part[wave][lane] = mine;
+    __syncthreads();
+    if (wave == 0 && lane < 32) {
+        const int n = nw * 32 + lane;
+        float total = bias ? h2f(bias[n]) : 0.f;
+        for (int w = 0; w < waves; ++w)
+            total += part[w][lane];
+        out[static_cast<size_t>(m) * N + n] = f2h(total);
+    }
+}
+
 template <typename LIdxT, typename RIdxT>
 __global__ void __launch_bounds__(256)
 sbvr_mm_T_kernel(const uint32_t *__restrict__ l_bvr, const void *__restrict__ l_idx,
@@ -1742,6 +1849,29 @@ int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_co
     if (idx_bytes != 1 && idx_bytes != 2)
         return fail(SBVR_HIP_EINVAL, "idx_bytes must be 1 or 2, got %d", idx_bytes);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (idx_bytes == 1 && L > 256)
+        return fail(SBVR_HIP_EINVAL, "uint8 indices cannot address L=%d lines", L);
+    if (M <= 65535 && (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) && reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0) {
+        // lanes along K; as many waves as there are steps of 64 rows, up to kRowDeqWaves
+        const int steps = (K + 63) / 64;
+        const int waves = steps < kRowDeqWaves ? steps : kRowDeqWaves;
+        const dim3 grid(static_cast<unsigned>(N / 32), static_cast<unsigned>(M)), block(64 * waves);
+#define SBVR_ROWDEQ(s)                                                                                            \
+    case s:                                                                                                       \
+        hipLaunchKernelGGL(sbvr_row_deq_lanes_kernel<s>, grid, block, 0, st, static_cast<const uint16_t *>(x), r_bvr, \
+                           r_coeff_idx, static_cast<const uint16_t *>(r_coeff_cache),                            \
+                           static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out), M, N, K, L, G,     \
+                           idx_bytes == 2 ? 1 : 0);                                                               \
+        break
+        switch (S) {
+            SBVR_ROWDEQ(2); SBVR_ROWDEQ(3); SBVR_ROWDEQ(4); SBVR_ROWDEQ(6); SBVR_ROWDEQ(8);
+        }
+#undef SBVR_ROWDEQ
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return fail(SBVR_HIP_ELAUNCH, "row_deq launch: %s", hipGetErrorString(e));
+        return SBVR_HIP_OK;
+    }
     const size_t total = static_cast<size_t>(M) * N;
     const dim3 grid(static_cast<unsigned>((total + 255) / 256)), block(256);
     if (idx_bytes == 1)

@@ -60,7 +60,10 @@ def test_mm_T_object_api(oracle, golden):
     assert np.abs(y.float().cpu().numpy() - w @ w.T).max() <= 1e-2 * np.abs(w @ w.T).max()
 
 
-@pytest.mark.parametrize("M,N,K,S,G,L", [(1, 256, 64, 4, 256, 9), (2, 512, 40, 2, 128, 300)])
+@pytest.mark.parametrize("M,N,K,S,G,L", [(1, 256, 64, 4, 256, 9), (2, 512, 40, 2, 128, 300),
+                                         (3, 1024, 4096, 4, 128, 256), (1, 96, 1000, 3, 32, 700),
+                                         (5, 64, 130, 8, 64, 40), (1, 4096, 2048, 6, 128, 256),
+                                         (2, 14336, 512, 4, 128, 256), (1, 32, 1, 4, 32, 2)])
 def test_row_deq_mm_T(oracle, M, N, K, S, G, L):
     import sbvr
     dev = torch.device("cuda:0")
