@@ -270,9 +270,12 @@ __device__ __forceinline__ float wave_fsum(float v)
 //   kXAddNorm M == 1: r = fp16(x + delta), weight * fp16(r * rsqrt(mean(r^2) + eps)),
 //             the decoder layer's residual add followed by its RMSNorm
 //             (models/sbvr_llama.py:396-400 and :118-124); every workgroup works out
-//             the mean over all of K by itself, workgroup (0, 0) writes r to x_out.
-constexpr int kXPlain = 0, kXSwiGLU = 1, kXAddNorm = 2;
-constexpr int kNormChunksPerThread = 2;       // 16-byte chunks of x a thread sums for the norm
+//             the mean over all of K by itself: its threads share out x and delta in
+//             16-byte chunks (one each, or two each with kXAddNorm2), leave r in LDS,
+//             where the waves then find their own elements; workgroup (0, 0) writes r
+//             to x_out.
+constexpr int kXPlain = 0, kXSwiGLU = 1, kXAddNorm = 2, kXAddNorm2 = 3;   // (3: two chunks of x per thread for the norm)
+constexpr int kNormChunksMax = 2;             // 16-byte chunks of x a thread sums for the norm, at most
 
 __device__ __forceinline__ uint32_t swiglu_pair(uint32_t g, uint32_t u)
 {
@@ -350,39 +353,40 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     SBVR_STAMP(0);
     // -- 1. requests.  Unit u = (sub-group u / CT, column tile u % CT).
     constexpr int U = SP * CT;
+    constexpr bool kNorm = XM == kXAddNorm || XM == kXAddNorm2;
+    constexpr int NV = XM == kXAddNorm2 ? 2 : 1;                        // chunks of x and of delta per thread
     uint32_t xx[SP][MT][4];
-    uint32_t x2[XM == kXPlain ? 1 : SP][XM == kXPlain ? 1 : MT][4];     // up (SwiGLU), delta (add + norm)
-    uint32_t xw[XM == kXAddNorm ? SP : 1];                              // norm weights
-    v4u sx[kNormChunksPerThread], sd[kNormChunksPerThread];             // this thread's share of all of x and delta
-#pragma unroll
-    for (int sgi = 0; sgi < SP; ++sgi)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                xx[sgi][mt][r] = 0u;
-                if constexpr (XM != kXPlain)
-                    x2[sgi][mt][r] = 0u;
-                if (XM != kXPlain ? mt * 4 + r < 1 : mt * 4 + r < a.M) {    // wave-uniform; one row with a prologue
-                    const size_t at = static_cast<size_t>(mt * 4 + r) * a.xstride + static_cast<size_t>(sg0 + sgi) * kSub;
-                    xx[sgi][mt][r] = reinterpret_cast<const uint32_t *>(a.x + at)[lane];
-                    if constexpr (XM == kXSwiGLU)
-                        x2[sgi][mt][r] = reinterpret_cast<const uint32_t *>(a.x + at + K)[lane];
-                    if constexpr (XM == kXAddNorm)
-                        x2[sgi][mt][r] = reinterpret_cast<const uint32_t *>(a.delta + at)[lane];
-                }
-            }
-    if constexpr (XM == kXAddNorm) {
+    uint32_t x2[XM == kXSwiGLU ? SP : 1][XM == kXSwiGLU ? MT : 1][4];   // up (SwiGLU)
+    uint32_t xw[kNorm ? SP : 1];                                        // norm weights
+    v4u sx[NV], sd[NV];                                                 // this thread's share of all of x and delta
+    if constexpr (!kNorm) {
 #pragma unroll
         for (int sgi = 0; sgi < SP; ++sgi)
-            xw[sgi] = reinterpret_cast<const uint32_t *>(a.norm_w + static_cast<size_t>(sg0 + sgi) * kSub)[lane];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    xx[sgi][mt][r] = 0u;
+                    if constexpr (XM == kXSwiGLU)
+                        x2[sgi][mt][r] = 0u;
+                    if (XM != kXPlain ? mt * 4 + r < 1 : mt * 4 + r < a.M) {    // wave-uniform; one row with a prologue
+                        const size_t at = static_cast<size_t>(mt * 4 + r) * a.xstride + static_cast<size_t>(sg0 + sgi) * kSub;
+                        xx[sgi][mt][r] = reinterpret_cast<const uint32_t *>(a.x + at)[lane];
+                        if constexpr (XM == kXSwiGLU)
+                            x2[sgi][mt][r] = reinterpret_cast<const uint32_t *>(a.x + at + K)[lane];
+                    }
+                }
+    } else {
         // (never conditional: a chunk past the end repeats the last one and is left out of the sum)
 #pragma unroll
-        for (int j = 0; j < kNormChunksPerThread; ++j) {
+        for (int j = 0; j < NV; ++j) {
             const int c = min(tid + j * static_cast<int>(blockDim.x), (K >> 3) - 1);
             sx[j] = reinterpret_cast<const v4u *>(a.x)[c];
             sd[j] = reinterpret_cast<const v4u *>(a.delta)[c];
         }
+#pragma unroll
+        for (int sgi = 0; sgi < SP; ++sgi)
+            xw[sgi] = reinterpret_cast<const uint32_t *>(a.norm_w + static_cast<size_t>(sg0 + sgi) * kSub)[lane];
     }
     // line indices: one load per sub-group, lane l takes the index of column n_base + l of the
     // window (16*CT <= 64 columns); they are handed to the (tile, column) lanes later, in LDS
@@ -417,12 +421,15 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     //       lane then reads its 32 bytes back.  Row tiles go from the last one,
     //       the only one that may have fewer than 4 rows, to the first, so a row
     //       of the buffer that is not rewritten holds zeros.
-    float inv = 0.f;             // XM == kXAddNorm: rsqrt(mean((x + delta)^2) + eps)
-    if constexpr (XM == kXAddNorm) {
+    float inv = 0.f;             // with the norm: rsqrt(mean((x + delta)^2) + eps)
+    if constexpr (kNorm) {
         float ss = 0.f;
+        float *const sums = reinterpret_cast<float *>(smem + waves * 2048);
+        v4u *const rbuf = reinterpret_cast<v4u *>(smem + waves * 2048 + 64);      // r = fp16(x + delta), all of K
 #pragma unroll
-        for (int j = 0; j < kNormChunksPerThread; ++j) {
-            const bool counts = tid + j * static_cast<int>(blockDim.x) < (K >> 3);
+        for (int j = 0; j < NV; ++j) {
+            const int c = tid + j * static_cast<int>(blockDim.x);
+            const bool counts = c < (K >> 3);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const uint32_t r = add_pair(sx[j][e], sd[j][e]);
@@ -430,9 +437,10 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
                 const float lo = h2f(static_cast<uint16_t>(r & 0xffffu)), hi = h2f(static_cast<uint16_t>(r >> 16));
                 ss += counts ? fmaf(lo, lo, hi * hi) : 0.f;
             }
+            if (counts)
+                rbuf[c] = sx[j];
         }
         ss = wave_fsum(ss);
-        float *const sums = reinterpret_cast<float *>(smem + waves * 2048);
         if (lane == 0)
             sums[wave] = ss;
         __syncthreads();
@@ -440,6 +448,16 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
         for (int w = 0; w < waves; ++w)
             total += sums[w];
         inv = rsqrtf(total / static_cast<float>(K) + a.eps);
+        // the wave's own elements of r (batch row 0)
+#pragma unroll
+        for (int sgi = 0; sgi < SP; ++sgi) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    xx[sgi][mt][r] = 0u;
+            xx[sgi][0][0] = reinterpret_cast<const uint32_t *>(rbuf)[(sg0 + sgi) * (kSub / 2) + lane];
+        }
     }
     v8i A[SP][MT];
     float scale[SP][MT];         // of this lane's batch row (blk)
@@ -460,8 +478,8 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
                         uint32_t v = xx[sgi][mt][r];
                         if constexpr (XM == kXSwiGLU)
                             v = swiglu_pair(v, x2[sgi][mt][r]);
-                        if constexpr (XM == kXAddNorm)
-                            v = norm_pair(add_pair(v, x2[sgi][mt][r]), xw[sgi], inv);
+                        if constexpr (kNorm)
+                            v = norm_pair(v, xw[sgi], inv);
                         // 2^e puts the largest magnitude of the sub-group into [32, 64)
                         // (fp16 bits order like magnitudes; subnormals count as 2^-15)
                         const uint32_t amax = wave_umax(max(v & 0x7fffu, (v >> 16) & 0x7fffu));
@@ -623,10 +641,10 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
             r = hadd(r, a.bias[n]);
         a.out[at] = r;
     }
-    if constexpr (XM == kXAddNorm) {
+    if constexpr (kNorm) {
         if (blockIdx.x == 0 && blockIdx.y == 0) {
 #pragma unroll
-            for (int j = 0; j < kNormChunksPerThread; ++j) {
+            for (int j = 0; j < NV; ++j) {
                 const int c = tid + j * static_cast<int>(blockDim.x);
                 if (c < (K >> 3))
                     reinterpret_cast<v4u *>(a.x_out)[c] = sx[j];
@@ -754,6 +772,8 @@ hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, int xm, hipStrea
         return p.MT == 1 ? launch_gemv_shape<S, 1, kXSwiGLU>(a, p, st) : hipErrorInvalidConfiguration;
     if (xm == kXAddNorm)
         return p.MT == 1 ? launch_gemv_shape<S, 1, kXAddNorm>(a, p, st) : hipErrorInvalidConfiguration;
+    if (xm == kXAddNorm2)
+        return p.MT == 1 ? launch_gemv_shape<S, 1, kXAddNorm2>(a, p, st) : hipErrorInvalidConfiguration;
     switch (p.MT) {
     case 1: return launch_gemv_shape<S, 1, kXPlain>(a, p, st);
 #ifndef SBVR_FAST_BUILD
@@ -1722,13 +1742,17 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         return SBVR_HIP_OK;
     }
     if ((!(flags & 1) || pro.mode != kXPlain) && aligned && mfma_path_ok(M, N, K, S, G)) {
-        // add + norm: the workgroup's threads share out all of K, kNormChunksPerThread chunks of 8 each
-        const int min_waves = pro.mode == kXAddNorm ? (K / 8 + 64 * kNormChunksPerThread - 1) / (64 * kNormChunksPerThread) : 1;
+        // add + norm: the threads of a workgroup share out all of K, at most kNormChunksMax chunks of 8 each
+        const int min_waves = pro.mode == kXAddNorm ? (K / 8 + 64 * kNormChunksMax - 1) / (64 * kNormChunksMax) : 1;
         GemvPlan p = plan_gemv(M, N, K, S, current_cus(), min_waves);
         if (p.CT == 0 && pro.mode != kXPlain)
             return fail(SBVR_HIP_EUNSUPPORTED, "no launch shape for the fused prologue (K=%d)", K);
-        if (pro.mode == kXAddNorm)
-            p.lds += 64;          // one partial sum of squares per wave
+        int xm = pro.mode;
+        if (pro.mode == kXAddNorm) {
+            p.lds += 64 + static_cast<size_t>(K) * 2;          // one partial sum of squares per wave, and fp16(x + delta)
+            if (K / 8 > 64 * p.waves)
+                xm = kXAddNorm2;                                 // two chunks of x per thread
+        }
         if (p.CT > 0) {
         if (env_int("SBVR_HIP_SHOW_PLAN", 0))
             fprintf(stderr, "sbvr_hip plan M=%d N=%d K=%d S=%d: CT=%d SP=%d MT=%d waves=%d wgs=%d ksplit=%d\n", M, N, K, S, p.CT, p.SP, p.MT, p.waves, p.n_wgs, p.ksplit);
@@ -1759,7 +1783,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
                 return fail(SBVR_HIP_EINVAL, "workspace must be 8-byte aligned");
             a.acc = static_cast<unsigned long long *>(workspace);
         }
-        const hipError_t e = launch_gemv(S, a, p, pro.mode, st);
+        const hipError_t e = launch_gemv(S, a, p, xm, st);
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "gemv launch (CT=%d SP=%d MT=%d waves=%d ksplit=%d): %s", p.CT, p.SP, p.MT, p.waves, p.ksplit, hipGetErrorString(e));
         return SBVR_HIP_OK;
