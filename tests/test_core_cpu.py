@@ -177,3 +177,22 @@ def test_argument_validation_without_gpu():
     assert rc == -1
     rc = lib.sbvr_hip_row_deq_mm_T(p, p, p, 1, p, None, p, 1, 48, 64, 4, 32, 4, None)
     assert rc == -1        # N must be a multiple of 32 and of G
+
+
+def test_torch_extension_mirrors_the_reference_operators():
+    """The compiled PyTorch extension (csrc/sbvr_ops_hip.cpp) offers the reference's operator
+    names (sbvr_ops.cpp:152-172) and refuses CPU tensors, like the ctypes binding."""
+    import torch
+    from sbvr import _sbvr_hip_ops as ops, hip
+    for name in ("_sbvr_mm_T", "_sbvr_row_deq_mm_T", "_sbvr_cuda_init", "_sbvr_hip_init", "_sbvr_linear_f16",
+                 "_sbvr_linear_f16_swiglu", "_sbvr_linear_f16_add_rmsnorm"):
+        assert callable(getattr(ops, name)), name
+    assert ops.version() == hip._load().sbvr_hip_version()
+    x = torch.zeros((1, 128), dtype=torch.float16)
+    bvr = torch.zeros((4, 16, 4), dtype=torch.uint32)
+    idx = torch.zeros((1, 16), dtype=torch.uint8)
+    cache = torch.zeros((4, 4), dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="must be on a GPU"):
+        ops._sbvr_linear_f16(x, bvr, idx, cache)
+    with pytest.raises(RuntimeError, match="must be on a GPU"):
+        ops._sbvr_mm_T(bvr, idx, cache, bvr, idx, cache, torch.zeros(0, dtype=torch.float16))

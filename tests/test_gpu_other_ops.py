@@ -132,3 +132,42 @@ def test_hip_init_and_bad_arguments():
                               bvr, idx, cache, None, 128)                                  # not contiguous
     with pytest.raises(TypeError):
         sbvr._sbvr_linear_f16(x, bvr, idx.to(torch.uint16), cache, None, 128)          # 16 lines want uint8
+
+
+def test_torch_extension_equals_ctypes_binding(oracle):
+    """Both bindings call the same entry points: identical bits, on the caller's stream."""
+    import sbvr
+    from sbvr import _sbvr_hip_ops as ops, synth
+    dev = torch.device("cuda:0")
+    ops._sbvr_hip_init()
+    none = torch.zeros(0, dtype=torch.float16, device=dev)
+    for (M, N, K, S, L) in [(1, 4096, 4096, 4, 256), (3, 1000, 1024, 3, 300), (48, 512, 1024, 4, 64)]:
+        bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(N, K, S, 128, L, seed=N))
+        x = torch.randn((M, K), generator=torch.Generator().manual_seed(K)).to(torch.float16).to(dev)
+        bias = torch.randn((N,), generator=torch.Generator().manual_seed(1)).to(torch.float16).to(dev)
+        assert torch.equal(ops._sbvr_linear_f16(x, bvr, idx, cache), sbvr._sbvr_linear_f16(x, bvr, idx, cache))
+        assert torch.equal(ops._sbvr_linear_f16(x, bvr, idx, cache, bias, 128),
+                           sbvr._sbvr_linear_f16(x, bvr, idx, cache, bias, 128))
+    # the reference's two operator forms, reference argument lists
+    lb, li, lc = (t.to(dev) for t in synth.random_encoding(2, 1024, 4, 128, 16, seed=3))
+    rb, ri, rc = (t.to(dev) for t in synth.random_encoding(640, 1024, 4, 128, 256, seed=4))
+    assert torch.equal(ops._sbvr_mm_T(lb, li, lc, rb, ri, rc, none), sbvr._sbvr_mm_T(lb, li, lc, rb, ri, rc, none))
+    tb, ti, tc = (t.to(dev) for t in synth.random_encoding(1024, 640, 4, 128, 256, seed=5))      # W^T: (K, N)
+    x = torch.randn((2, 1024), generator=torch.Generator().manual_seed(6)).to(torch.float16).to(dev)
+    assert torch.equal(ops._sbvr_row_deq_mm_T(x, tb, ti, tc, none, 0), sbvr._sbvr_row_deq_mm_T(x, tb, ti, tc, none, 0))
+    # one-row variants
+    bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(512, 1024, 4, 128, 256, seed=7))
+    gu = torch.randn((1, 2048), generator=torch.Generator().manual_seed(8)).to(torch.float16).to(dev)
+    assert torch.equal(ops._sbvr_linear_f16_swiglu(gu, bvr, idx, cache), sbvr._sbvr_linear_f16_swiglu(gu, bvr, idx, cache))
+    x1, d1 = x[:1].contiguous(), x[1:].contiguous()
+    w = torch.ones(1024, dtype=torch.float16, device=dev)
+    xo1, xo2 = torch.empty_like(x1), torch.empty_like(x1)
+    a = ops._sbvr_linear_f16_add_rmsnorm(x1, d1, w, 1e-5, xo1, bvr, idx, cache)
+    b = sbvr._sbvr_linear_f16_add_rmsnorm(x1, d1, w, 1e-5, xo2, bvr, idx, cache)
+    assert torch.equal(a, b) and torch.equal(xo1, xo2)
+    # on a side stream the extension launches there too
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        y = ops._sbvr_linear_f16(x, bvr, idx, cache)
+    side.synchronize()
+    assert torch.equal(y, sbvr._sbvr_linear_f16(x, bvr, idx, cache))
