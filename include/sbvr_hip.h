@@ -30,7 +30,7 @@ extern "C" {
 #define SBVR_HIP_ELAUNCH (-3)     /* HIP reported an error at launch */
 #define SBVR_HIP_EWORKSPACE (-4)  /* workspace missing or too small */
 
-/* ABI version of this header (major*100 + minor). */
+/* ABI version of this header (major*100 + minor); 101 added the one-row linears with a fused prologue. */
 int sbvr_hip_version(void);
 
 /* Text of the last error raised on this thread ("" if none). */

@@ -1646,7 +1646,7 @@ extern "C" {
 void sbvr_hip_debug_set_trace(unsigned long long *p) { g_trace = p; }
 #endif
 
-int sbvr_hip_version(void) { return 100; }
+int sbvr_hip_version(void) { return 101; }      // 101: the one-row linears with a fused prologue
 
 const char *sbvr_hip_last_error(void) { return g_err; }
 
