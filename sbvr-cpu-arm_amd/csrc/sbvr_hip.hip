@@ -1509,13 +1509,15 @@ sbvr_mm_T_kernel(const uint32_t *__restrict__ l_bvr, const void *__restrict__ l_
 
 // Both operands encoded (the form the reference's kernels compute, sbvr_kernel.cu:464-562
 // and sbvr_kernel.cpp:251-399): out[m,n] = sum_g sum_{l,r} popcount_g(L_l & R_r) a_l b_r.
-// Lane = column, so a wave reads 64 * SR consecutive plane words per word of K (coalesced)
-// while the left operand's words and coefficients are wave-uniform (scalar loads).  The
+// A wave owns 64 / Q columns and Q parts of its share of K: lane = part * (64 / Q) + column,
+// so it reads Q runs of (64 / Q) * SR consecutive plane words per word of K.  With Q = 1 the
+// left operand's words and coefficients are wave-uniform (scalar loads); Q = 4 is for
+// matrices with so few columns that 64-column workgroups would leave most CUs idle.  The
 // waves of a workgroup split the groups of K and meet in LDS; blockIdx.y is the left row.
 // Popcounts are exact integers per group; coefficients are applied in fp32.
 constexpr int kPopcWaves = 8, kPopcChunk = 8;      // words of K whose plane words a lane holds at once
 
-template <int SL, int SR>
+template <int SL, int SR, int Q>
 __global__ void __launch_bounds__(64 * kPopcWaves)
 sbvr_mm_T_popc_kernel(const uint32_t *__restrict__ l_bvr, const uint8_t *__restrict__ l_idx, int l_idx16,
                       const uint16_t *__restrict__ l_cache, const uint32_t *__restrict__ r_bvr,
@@ -1523,15 +1525,17 @@ sbvr_mm_T_popc_kernel(const uint32_t *__restrict__ l_bvr, const uint8_t *__restr
                       const uint16_t *__restrict__ bias, uint16_t *__restrict__ out,
                       int M, int N, int K, int wpg, int Ll, int Lr)
 {
-    __shared__ float red[kPopcWaves][64];
+    constexpr int C = 64 / Q;                       // columns of a wave
+    __shared__ float red[kPopcWaves][C];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int m = blockIdx.y;
-    const int n = blockIdx.x * 64 + lane, n_ld = min(n, N - 1);
+    const int col = lane & (C - 1), part = lane / C;
+    const int n = blockIdx.x * C + col, n_ld = min(n, N - 1);
     const int words = K / 32;
     const int chunks = (words + kPopcChunk - 1) / kPopcChunk;
-    const int cpw = (chunks + kPopcWaves - 1) / kPopcWaves;         // chunks per wave
-    const int c_begin = wave * cpw, c_end = min(chunks, c_begin + cpw);
+    const int cpw = (chunks + kPopcWaves * Q - 1) / (kPopcWaves * Q);     // chunks per (wave, part)
+    const int c_begin = (wave * Q + part) * cpw, c_end = min(chunks, c_begin + cpw);      // per lane when Q > 1
 
     auto load_chunk = [&](int c, uint32_t (&rw)[kPopcChunk][SR], int (&line)[kPopcChunk]) __attribute__((always_inline)) {
 #pragma unroll
@@ -1551,7 +1555,8 @@ sbvr_mm_T_popc_kernel(const uint32_t *__restrict__ l_bvr, const uint8_t *__restr
     float acc = 0.f;
     uint32_t rw0[kPopcChunk][SR], rw1[kPopcChunk][SR];
     int ln0[kPopcChunk], ln1[kPopcChunk];
-    auto compute = [&](int c, const uint32_t (&rw)[kPopcChunk][SR], const int (&line)[kPopcChunk]) __attribute__((always_inline)) {
+    // one chunk; `live` is false for a chunk past the lane's range (its counts are then masked out)
+    auto compute = [&](int c, bool live, const uint32_t (&rw)[kPopcChunk][SR], const int (&line)[kPopcChunk]) __attribute__((always_inline)) {
         int cnt[SL][SR];
 #pragma unroll
         for (int l = 0; l < SL; ++l)
@@ -1561,20 +1566,30 @@ sbvr_mm_T_popc_kernel(const uint32_t *__restrict__ l_bvr, const uint8_t *__restr
 #pragma unroll
         for (int i = 0; i < kPopcChunk; ++i) {
             const int w = c * kPopcChunk + i;
-            if (w >= words)                                          // wave-uniform
-                break;
-            const uint32_t *lp = l_bvr + (static_cast<size_t>(w) * M + m) * SL;       // wave-uniform
+            if constexpr (Q == 1) {
+                if (w >= words)                                      // wave-uniform
+                    break;
+            }
+            const bool counts = Q == 1 || (live && w < words);
+            const int wl = Q == 1 ? w : min(w, words - 1);
+            const uint32_t *lp = l_bvr + (static_cast<size_t>(wl) * M + m) * SL;      // wave-uniform when Q == 1
 #pragma unroll
             for (int l = 0; l < SL; ++l) {
-                const uint32_t lw = __builtin_amdgcn_readfirstlane(lp[l]);
+                uint32_t lw = lp[l];
+                if constexpr (Q == 1)
+                    lw = __builtin_amdgcn_readfirstlane(lw);
+                else
+                    lw = counts ? lw : 0u;
 #pragma unroll
                 for (int r = 0; r < SR; ++r)
                     cnt[l][r] += __builtin_popcount(lw & rw[i][r]);
             }
             if ((i + 1) % wpg == 0) {                                // wave-uniform: last word of its group
-                const size_t lat = (static_cast<size_t>(w / wpg) * M + m) << l_idx16;
+                const size_t lat = (static_cast<size_t>(wl / wpg) * M + m) << l_idx16;
                 const int llo = l_idx[lat], lhi = l_idx[lat + l_idx16];
-                const int lline = __builtin_amdgcn_readfirstlane(min(l_idx16 ? llo | (lhi << 8) : llo, Ll - 1));
+                int lline = min(l_idx16 ? llo | (lhi << 8) : llo, Ll - 1);
+                if constexpr (Q == 1)
+                    lline = __builtin_amdgcn_readfirstlane(lline);
                 const uint16_t *ca = l_cache + static_cast<size_t>(lline) * SL;
                 const int rline = min(r_idx16 ? (line[i] & 0xff) | ((line[i] >> 8) & 0xff00) : line[i] & 0xff, Lr - 1);
                 const uint16_t *cb = r_cache + static_cast<size_t>(rline) * SR;
@@ -1594,23 +1609,40 @@ sbvr_mm_T_popc_kernel(const uint32_t *__restrict__ l_bvr, const uint8_t *__restr
         }
     };
 
-    if (c_begin < c_end) {
-        load_chunk(c_begin, rw0, ln0);
-        for (int c = c_begin; c < c_end; c += 2) {
-            load_chunk(min(c + 1, chunks - 1), rw1, ln1);
-            compute(c, rw0, ln0);
-            load_chunk(min(c + 2, chunks - 1), rw0, ln0);
-            if (c + 1 < c_end)
-                compute(c + 1, rw1, ln1);
+    if constexpr (Q == 1) {
+        if (c_begin < c_end) {
+            load_chunk(c_begin, rw0, ln0);
+            for (int c = c_begin; c < c_end; c += 2) {
+                load_chunk(min(c + 1, chunks - 1), rw1, ln1);
+                compute(c, true, rw0, ln0);
+                load_chunk(min(c + 2, chunks - 1), rw0, ln0);
+                if (c + 1 < c_end)
+                    compute(c + 1, true, rw1, ln1);
+            }
         }
+    } else {
+        // the parts of a wave walk their ranges in step: same trip count for every lane
+        load_chunk(min(c_begin, chunks - 1), rw0, ln0);
+        for (int t = 0; t < cpw; t += 2) {
+            const int c = c_begin + t;
+            load_chunk(min(c + 1, chunks - 1), rw1, ln1);
+            compute(c, c < c_end, rw0, ln0);
+            load_chunk(min(c + 2, chunks - 1), rw0, ln0);
+            if (t + 1 < cpw)
+                compute(c + 1, c + 1 < c_end, rw1, ln1);
+        }
+#pragma unroll
+        for (int off = C; off < 64; off <<= 1)
+            acc += __shfl_xor(acc, off, 64);
     }
-    red[wave][lane] = acc;
+    if (part == 0)
+        red[wave][col] = acc;
     __syncthreads();
-    if (wave == 0 && n < N) {
+    if (wave == 0 && part == 0 && n < N) {
         float total = 0.f;
 #pragma unroll
         for (int w = 0; w < kPopcWaves; ++w)
-            total += red[w][lane];
+            total += red[w][col];
         uint16_t res = f2h(total);
         if (bias)
             res = hadd(res, bias[n]);
@@ -1619,14 +1651,22 @@ sbvr_mm_T_popc_kernel(const uint32_t *__restrict__ l_bvr, const uint8_t *__restr
 }
 
 template <int SL>
-bool launch_mm_T_popc_sr(int Sr, dim3 grid, hipStream_t st, const uint32_t *l_bvr, const uint8_t *l_idx, int l16,
+bool launch_mm_T_popc_sr(int Sr, int Q, hipStream_t st, const uint32_t *l_bvr, const uint8_t *l_idx, int l16,
                          const uint16_t *lc, const uint32_t *r_bvr, const uint8_t *r_idx, int r16, const uint16_t *rc,
                          const uint16_t *b, uint16_t *o, int M, int N, int K, int wpg, int Ll, int Lr)
 {
     const dim3 block(64 * kPopcWaves);
-#define SBVR_POPC(SR)                                                                                              \
-    hipLaunchKernelGGL((sbvr_mm_T_popc_kernel<SL, SR>), grid, block, 0, st, l_bvr, l_idx, l16, lc, r_bvr, r_idx, \
-                       r16, rc, b, o, M, N, K, wpg, Ll, Lr)
+    const int cols = 64 / Q;
+    const dim3 grid(static_cast<unsigned>((N + cols - 1) / cols), static_cast<unsigned>(M));
+#define SBVR_POPC(SR)                                                                                                \
+    do {                                                                                                             \
+        if (Q == 4)                                                                                                  \
+            hipLaunchKernelGGL((sbvr_mm_T_popc_kernel<SL, SR, 4>), grid, block, 0, st, l_bvr, l_idx, l16, lc, r_bvr, \
+                               r_idx, r16, rc, b, o, M, N, K, wpg, Ll, Lr);                                          \
+        else                                                                                                         \
+            hipLaunchKernelGGL((sbvr_mm_T_popc_kernel<SL, SR, 1>), grid, block, 0, st, l_bvr, l_idx, l16, lc, r_bvr, \
+                               r_idx, r16, rc, b, o, M, N, K, wpg, Ll, Lr);                                          \
+    } while (0)
     switch (Sr) {
     case 2: SBVR_POPC(2); return true;
     case 3: SBVR_POPC(3); return true;
@@ -1936,7 +1976,10 @@ int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_byte
     const int wpg = G / 32;
     if (M <= 64 && (wpg == 1 || wpg == 2 || wpg == 4 || wpg == 8) && Sl >= 2 && Sl <= 4 &&
         reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0 && static_cast<double>(K / 32) * N * Sr < 2147483648.0) {
-        const dim3 pgrid(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(M));
+        // 16-column windows (four parts of K inside a wave) when 64-column ones would leave half the CUs without a
+        // workgroup: measured 13 us against 27 us at N=4096, K=14336, but 26 us against 11.5 us at N=14336, K=4096
+        const int eq = env_int("SBVR_HIP_POPC_Q", 0);
+        const int pgrid = eq ? eq : (static_cast<long>((N + 63) / 64) * M * 2 <= current_cus() ? 4 : 1);
         const uint8_t *li = static_cast<const uint8_t *>(l_coeff_idx), *ri = static_cast<const uint8_t *>(r_coeff_idx);
         const int l16 = l_idx_bytes == 2, r16 = r_idx_bytes == 2;
         bool done = false;
