@@ -55,6 +55,21 @@ int sbvr_hip_dec_argmax_advance_f16(const void *logits, int n, long long *token,
                                     int max_seq, const float *cos_table, const float *sin_table, int head_dim,
                                     float *rot_now, void *stream);
 
+/* The end of a decode step in one launch: the final residual add and RMSNorm (as
+ * sbvr_hip_dec_add_rmsnorm_f16, delta may be NULL, x is not written), the fp16
+ * output head logits[v] = fp16(h . head[v]) for head (vocab, K) row-major
+ * (reference models/sbvr_llama.py:851-853, lm_head over the last hidden state;
+ * fp32 sums, one rounding), and the greedy choice and bookkeeping of
+ * sbvr_hip_dec_argmax_advance_f16 on those fp16 logits.  logits may be NULL
+ * (not stored).  K must be 512, 1024, 2048, 4096 or 8192 (-2 otherwise: run the
+ * three steps separately); x, delta, norm_weight and head 16-byte aligned.
+ * workspace: 16 bytes of device memory, zero-filled once; every launch leaves it
+ * zero-filled.  Launches that share a workspace must not overlap in time. */
+int sbvr_hip_dec_head_argmax_f16(const void *x, const void *delta, const void *norm_weight, float eps, const void *head,
+                                 int vocab, int K, void *logits, long long *token, long long *generated, long long *pos,
+                                 int max_seq, const float *cos_table, const float *sin_table, int head_dim,
+                                 float *rot_now, void *workspace, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

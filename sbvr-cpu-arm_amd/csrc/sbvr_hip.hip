@@ -25,11 +25,19 @@
 // 64-bit fixed-point accumulators (exact, so the result does not depend on
 // the order of arrival).
 //
-// Prefill path (M > 16), sbvr_gemm_mfma_kernel: weights decoded to fp16 tiles
-// in LDS, fp16 MFMA, fp32 accumulation.
+// For one batch row the kernel can take the elementwise step in front of the
+// linear along (SiLU(gate) * up, or residual add + RMSNorm) while it turns the
+// activations into A operands: sbvr_hip_linear_f16_swiglu / _add_rmsnorm.
 //
-// Portable kernels (any shape, one thread per output) back both, and serve the
-// trans=True and both-operands-encoded forms of the reference's operators.
+// Prefill path (M > 32), sbvr_gemm_mfma_kernel: weights decoded to fp16 tiles
+// in LDS, fp16 MFMA, fp32 accumulation; sbvr_gemm_rows32_kernel for 9..32 rows
+// (the batch rows are the 32 rows of one MFMA, weights decoded in registers).
+//
+// The reference's own operator forms: sbvr_mm_T_popc_kernel (both operands
+// encoded: popcounts per group, lane per column) and sbvr_row_deq_lanes_kernel
+// (trans=True weight, lanes along K).
+//
+// Portable kernels (any shape, one thread per output) back all of them.
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdint.h>
@@ -196,30 +204,39 @@ struct Planes {
     uint32_t w[S];
 };
 
-template <int S>
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+
+// The S plane words of one (word of K, column) pair.  kStream: non-temporal loads, for kernels that
+// read every plane word once per launch and are bound by that stream (measured on the decode kernel:
+// 8.3 us instead of 8.8 us at the 4096 -> 14336 shape, 13.5 instead of 14.5 us at 4096 -> 28672; the
+// 32-row, row-dequant and popcount kernels, bound by their arithmetic, gain nothing from it).
+template <int S, bool kStream = false>
 __device__ __forceinline__ Planes<S> load_planes(const uint32_t *p)
 {
+    auto ld4 = [](const uint32_t *q) __attribute__((always_inline)) -> v4u {
+        return kStream ? __builtin_nontemporal_load(reinterpret_cast<const v4u *>(q)) : *reinterpret_cast<const v4u *>(q);
+    };
+    auto ld2 = [](const uint32_t *q) __attribute__((always_inline)) -> v2u {
+        return kStream ? __builtin_nontemporal_load(reinterpret_cast<const v2u *>(q)) : *reinterpret_cast<const v2u *>(q);
+    };
     Planes<S> r;
     if constexpr (S == 4) {
-        const uint4 v = *reinterpret_cast<const uint4 *>(p);
+        const v4u v = ld4(p);
         r.w[0] = v.x; r.w[1] = v.y; r.w[2] = v.z; r.w[3] = v.w;
     } else if constexpr (S == 2) {
-        const uint2 v = *reinterpret_cast<const uint2 *>(p);
+        const v2u v = ld2(p);
         r.w[0] = v.x; r.w[1] = v.y;
     } else if constexpr (S == 8) {
-        const uint4 v0 = reinterpret_cast<const uint4 *>(p)[0];
-        const uint4 v1 = reinterpret_cast<const uint4 *>(p)[1];
+        const v4u v0 = ld4(p), v1 = ld4(p + 4);
         r.w[0] = v0.x; r.w[1] = v0.y; r.w[2] = v0.z; r.w[3] = v0.w;
         r.w[4] = v1.x; r.w[5] = v1.y; r.w[6] = v1.z; r.w[7] = v1.w;
     } else if constexpr (S == 6) {
-        const uint2 v0 = reinterpret_cast<const uint2 *>(p)[0];
-        const uint2 v1 = reinterpret_cast<const uint2 *>(p)[1];
-        const uint2 v2 = reinterpret_cast<const uint2 *>(p)[2];
+        const v2u v0 = ld2(p), v1 = ld2(p + 2), v2 = ld2(p + 4);
         r.w[0] = v0.x; r.w[1] = v0.y; r.w[2] = v1.x; r.w[3] = v1.y; r.w[4] = v2.x; r.w[5] = v2.y;
     } else {
 #pragma unroll
         for (int j = 0; j < S; ++j)
-            r.w[j] = p[j];
+            r.w[j] = kStream ? __builtin_nontemporal_load(p + j) : p[j];
     }
     return r;
 }
@@ -410,7 +427,7 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint32_t *wrow = a.bvr + static_cast<size_t>(sg0 + u / CT) * 4 * N * S;     // wave-uniform
-            q[u] = load_planes<S>(wrow + lane_w + (u % CT) * 16 * S);
+            q[u] = load_planes<S, true>(wrow + lane_w + (u % CT) * 16 * S);
         }
     }
     __builtin_amdgcn_sched_barrier(0);       // every request is out before anything waits
@@ -897,7 +914,7 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
         auto request = [&](int t, uint32_t (&wr)[S], uint32_t (&cr)[CW]) __attribute__((always_inline)) {
             const int k0 = t * kGemmBK;
             const uint32_t *wp = a.bvr + (static_cast<size_t>(k0 / 32 + bw) * N + n_ld) * S;
-            const Planes<S> pl = load_planes<S>(wp);
+            const Planes<S> pl = load_planes<S>(wp);      // (cached: every row tile of the launch reads these again)
 #pragma unroll
             for (int j = 0; j < S; ++j)
                 wr[j] = pl.w[j];

@@ -113,6 +113,8 @@ class SbvrLlamaDecoder:
         self.tok = torch.zeros(1, dtype=torch.int64, device=dev)
         self.pos = torch.zeros(1, dtype=torch.int64, device=dev)
         self.generated = torch.zeros(max_seq, dtype=torch.int64, device=dev)
+        self.logits = torch.empty((1, s.vocab), dtype=torch.float16, device=dev)
+        self.head_ws = torch.zeros(2, dtype=torch.int64, device=dev)              # cross-workgroup argmax of the head kernel
         self.graph = None
         self.stream = torch.cuda.Stream(device=dev)
 
@@ -151,7 +153,8 @@ class SbvrLlamaDecoder:
         return logits
 
     def _step_fused(self):
-        """5 launches per layer: q|k|v (with the residual add and norm in front),
+        """One launch for the end of the step (final norm, head, argmax) where the
+        hidden size has a kernel, and 5 launches per layer: q|k|v (with the residual add and norm in front),
         attention, o, gate|up (same), down (with SiLU*up in front).  The residual
         stream alternates between two buffers: a linear reads one and writes the
         sum to the other, since its workgroups do not run in step."""
@@ -166,6 +169,11 @@ class SbvrLlamaDecoder:
             delta = layer["o"](ctx)
             gate_up = layer["gate_up"].after_add_rmsnorm(b, delta, layer["norm2"], s.rms_eps, a)
             delta = layer["down"].after_swiglu(gate_up)
+        if hip.dec_head_argmax_supported(s.hidden):
+            # final norm, head, argmax and position advance in one launch
+            hip.dec_head_argmax(a, delta, self.final_norm, s.rms_eps, self.lm_head, self.logits, self.tok,
+                                self.generated, self.pos, self.head_ws, self.cos, self.sin, self.rot_now)
+            return self.logits
         hip.dec_add_rmsnorm(a, delta, self.final_norm, self.h, s.rms_eps)
         logits = torch.matmul(self.h, self.lm_head.t())                 # (1, vocab)
         hip.dec_argmax_advance(logits, self.tok, self.generated, self.pos, self.cos, self.sin, self.rot_now)

@@ -56,6 +56,8 @@ def _load():
     lib.sbvr_hip_dec_attention_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
     lib.sbvr_hip_dec_silu_mul_f16.argtypes = [vp, vp, i, vp]
     lib.sbvr_hip_dec_argmax_advance_f16.argtypes = [vp, i, vp, vp, vp, i, vp, vp, i, vp, vp]
+    lib.sbvr_hip_dec_head_argmax_f16.argtypes = [vp, vp, vp, ctypes.c_float, vp, i, i, vp, vp, vp, vp, i, vp, vp, i,
+                                                 vp, vp, vp]
     _lib = lib
     return lib
 
@@ -337,3 +339,37 @@ def dec_argmax_advance(logits, token, generated, pos, cos=None, sin=None, rot_no
                                                         sin.data_ptr() if rot_now is not None else None, head_dim,
                                                         rot_now.data_ptr() if rot_now is not None else None,
                                                         _stream()), "argmax_advance")
+
+
+def dec_head_argmax_supported(hidden):
+    """Whether dec_head_argmax has a kernel for this hidden size."""
+    return hidden in (512, 1024, 2048, 4096, 8192)
+
+
+def dec_head_argmax(x, delta, weight, eps, head, logits, token, generated, pos, workspace, cos=None, sin=None,
+                    rot_now=None):
+    """Final residual add + RMSNorm, fp16 output head, argmax and position advance in one launch.
+    ``head`` (vocab, hidden) fp16; ``logits`` (vocab,) fp16 or None; ``workspace``: two int64 zeros."""
+    for t, name in ((x, "x"), (weight, "weight"), (head, "head")) + (((delta, "delta"),) if delta is not None else ()) \
+            + (((logits, "logits"),) if logits is not None else ()):
+        _want(t, name, torch.float16)
+    for t, name in ((token, "token"), (generated, "generated"), (pos, "pos"), (workspace, "workspace")):
+        _want(t, name, torch.int64)
+    vocab, hidden = head.shape
+    if x.numel() != hidden or weight.numel() != hidden or workspace.numel() < 2 or \
+            (logits is not None and logits.numel() != vocab):
+        raise SbvrHipError("dec_head_argmax: tensor shapes do not match the head")
+    head_dim = 0
+    if rot_now is not None:
+        for t, name in ((cos, "cos"), (sin, "sin"), (rot_now, "rot_now")):
+            _want(t, name, torch.float32)
+        head_dim = rot_now.numel()
+        if cos.shape != (generated.numel(), head_dim // 2) or sin.shape != cos.shape:
+            raise SbvrHipError("dec_head_argmax: rotary tables must be (max_seq, head_dim / 2)")
+    _dec_check(_load().sbvr_hip_dec_head_argmax_f16(
+        x.data_ptr(), delta.data_ptr() if delta is not None else None, weight.data_ptr(), float(eps), head.data_ptr(),
+        vocab, hidden, logits.data_ptr() if logits is not None else None, token.data_ptr(), generated.data_ptr(),
+        pos.data_ptr(), generated.numel(), cos.data_ptr() if rot_now is not None else None,
+        sin.data_ptr() if rot_now is not None else None, head_dim,
+        rot_now.data_ptr() if rot_now is not None else None, workspace.data_ptr(), _stream()), "head_argmax")
+    return logits

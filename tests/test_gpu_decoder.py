@@ -216,3 +216,105 @@ def test_argmax_advance_leaves_rotation():
             assert int(gen[start]) == 123
         r = min(start + 1, max_seq - 1)
         assert torch.equal(rot, torch.cat((cos[r], sin[r])))
+
+
+@pytest.mark.parametrize("hidden,vocab", [(512, 1000), (1024, 129), (4096, 128256), (2048, 5000), (8192, 300)])
+@pytest.mark.parametrize("with_delta", [True, False])
+def test_head_argmax_kernel(hidden, vocab, with_delta):
+    """Final norm + fp16 head + argmax + bookkeeping in one launch, against numpy; two launches in a row
+    (the second must find the workspace clean), equal maxima resolved to the lowest index."""
+    import torch
+    from sbvr import hip
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(hidden + vocab)
+    x = torch.randn(hidden, generator=gen).to(torch.float16)
+    delta = (torch.randn(hidden, generator=gen) * 0.5).to(torch.float16) if with_delta else None
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=gen)).to(torch.float16)
+    head = (torch.randn((vocab, hidden), generator=gen) * 0.05).to(torch.float16)
+    head[vocab // 3] = head[vocab - 2]                  # two identical rows: a tie somewhere (maybe at the top)
+    max_seq, head_dim = 16, 64
+    cos = torch.rand((max_seq, head_dim // 2)).to(dev)
+    sin = torch.rand((max_seq, head_dim // 2)).to(dev)
+    logits = torch.empty(vocab, dtype=torch.float16, device=dev)
+    tok = torch.zeros(1, dtype=torch.int64, device=dev)
+    generated = torch.full((max_seq,), -1, dtype=torch.int64, device=dev)
+    pos = torch.tensor([4], dtype=torch.int64, device=dev)
+    rot = torch.zeros(head_dim, dtype=torch.float32, device=dev)
+    ws = torch.zeros(2, dtype=torch.int64, device=dev)
+    xd, wd, hd = x.to(dev), w.to(dev), head.to(dev)
+    dd = delta.to(dev) if with_delta else None
+
+    r = (x.float() + (delta.float() if with_delta else 0.0)).to(torch.float16)
+    inv = 1.0 / np.sqrt(np.mean(r.double().numpy() ** 2) + 1e-5)
+    h = (w.float() * (r.float() * np.float32(inv)).to(torch.float16).float()).to(torch.float16)
+    want = head.double().numpy() @ h.double().numpy()
+
+    for launch in range(2):
+        hip.dec_head_argmax(xd, dd, wd, 1e-5, hd, logits, tok, generated, pos, ws, cos, sin, rot)
+        torch.cuda.synchronize()
+        got = logits.float().cpu().numpy().astype(np.float64)
+        scale = max(np.abs(want).max(), 1e-6)
+        assert np.abs(got - want).max() <= 4e-3 * scale, np.abs(got - want).max()
+        # the choice is the first maximum of the kernel's own fp16 logits
+        assert int(tok) == int(np.argmax(logits.float().cpu().numpy()))
+        assert int(pos) == 5 + launch and int(generated[4 + launch]) == int(tok)
+        assert torch.equal(rot, torch.cat((cos[5 + launch], sin[5 + launch])))
+        assert int(ws[0]) == 0 and int(ws[1]) == 0
+    # the input row is left alone
+    assert torch.equal(xd.cpu(), x)
+
+
+def test_head_argmax_tie_and_nan():
+    import torch
+    from sbvr import hip
+
+    dev = torch.device("cuda:0")
+    hidden, vocab = 512, 700
+    x = torch.ones(hidden, dtype=torch.float16, device=dev)
+    w = torch.ones(hidden, dtype=torch.float16, device=dev)
+    head = torch.zeros((vocab, hidden), dtype=torch.float16, device=dev)
+    head[600, 0] = 3.0
+    head[250, 1] = 3.0                                  # same logit as row 600: the lower index wins
+    head[10, 0] = float("nan")                          # a NaN logit never wins
+    tok = torch.zeros(1, dtype=torch.int64, device=dev)
+    generated = torch.zeros(8, dtype=torch.int64, device=dev)
+    pos = torch.zeros(1, dtype=torch.int64, device=dev)
+    ws = torch.zeros(2, dtype=torch.int64, device=dev)
+    hip.dec_head_argmax(x, None, w, 1e-5, head, None, tok, generated, pos, ws)
+    torch.cuda.synchronize()
+    assert int(tok) == 250 and int(pos) == 1
+
+
+def test_decoder_with_fused_head(oracle):
+    """A hidden size for which the end of the step is one launch (final norm + head + argmax)."""
+    import torch
+    from sbvr.decoder import LlamaShape, SbvrLlamaDecoder
+
+    shape = LlamaShape(hidden=512, layers=2, heads=8, kv_heads=2, head_dim=64, ffn=1024, vocab=777)
+    dec = SbvrLlamaDecoder(shape, "cuda:0", lines=64, max_seq=16, seed=11)
+    for layer in dec.layers:
+        for k in ("qkv", "o", "gate_up", "down"):
+            layer[k].cache.mul_(2.0)
+    tokens = [5, 700, 33, 0]
+    dec.reset()
+    got = []
+    with torch.cuda.stream(dec.stream):
+        for t in tokens:
+            dec.tok.fill_(t)
+            got.append(dec.step().float().cpu().numpy()[0].copy())
+    ref = dense_reference(dec, oracle, tokens)
+    picked = dec.generated[:len(tokens)].cpu().numpy()
+    for p in range(len(tokens)):
+        err = np.abs(got[p] - ref[p]).max() / np.abs(ref[p]).max()
+        assert err < 2e-2, f"step {p}: logits differ by {err:.3e} of the largest"
+        assert ref[p][picked[p]] >= ref[p].max() - 2e-2 * np.abs(ref[p]).max()
+    # graph replay gives the same tokens
+    eager = dec.generated[:len(tokens)].clone()
+    dec.capture()
+    with torch.cuda.stream(dec.stream):
+        for t in tokens:
+            dec.tok.fill_(t)
+            dec.graph.replay()
+        torch.cuda.synchronize()
+    assert torch.equal(dec.generated[:len(tokens)], eager)
