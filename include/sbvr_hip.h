@@ -42,8 +42,11 @@ int sbvr_hip_init(int device);
 
 /* Bytes of device workspace sbvr_hip_linear_f16 wants for this shape (0 if
  * none).  The workspace must be zero-filled once after allocation; every call
- * leaves it zero-filled where it needs zeros.  Calls that share a workspace
- * must not overlap in time. */
+ * leaves it zero-filled.  Calls that share a workspace must not overlap in
+ * time.  For up to 16 rows (decode kernel, K split across workgroups) the
+ * workspace is required; for more rows (prefill kernel with few output tiles)
+ * it is optional: without it that launch is not split along K, which is slower
+ * but gives the same result up to the order of the fp32 additions. */
 size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
 
 /*

@@ -854,6 +854,8 @@ struct GemmArgs {
     int M, N, K, L;
     int steps_per_group;   // G / 64
     int idx16;
+    int ksplit;            // workgroups along K (blockIdx.z); 1: results go straight to out
+    float *part;           // ksplit > 1: (ksplit, M, N) fp32 partial results, all zero between launches
 #ifdef SBVR_TRACE
     unsigned long long *trace;
 #endif
@@ -882,7 +884,8 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int N = a.N, K = a.K, M = a.M;
     const int n0 = blockIdx.x * kGemmBN, m0 = blockIdx.y * kGemmBM;
-    const int steps = K / kGemmBK;
+    const int steps = K / kGemmBK / a.ksplit;            // of this workgroup: tiles t_base .. t_base + steps - 1 of K
+    const int t_base = blockIdx.z * steps;
     const int rounds = (steps + 2) / 3;                  // both kinds of waves run 3 * rounds steps (same barriers)
 
     if (wave >= 4) {
@@ -902,7 +905,7 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
         // (two byte loads whatever the index width: a branch between a 16-bit and an 8-bit load
         // inside the loop would make every later wait a wait for all loads)
         auto load_line = [&](int t) __attribute__((always_inline)) -> int {
-            const size_t at = (static_cast<size_t>(t / a.steps_per_group) * N + n_ld) << a.idx16;
+            const size_t at = (static_cast<size_t>((t_base + t) / a.steps_per_group) * N + n_ld) << a.idx16;
             const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
             const int lo = ib[at], hi = ib[at + a.idx16];
             return lo | (hi << 16);          // raw bytes: put together where the index is used, not here,
@@ -912,7 +915,7 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
         };
         // global loads of tile t into one register set
         auto request = [&](int t, uint32_t (&wr)[S], uint32_t (&cr)[CW]) __attribute__((always_inline)) {
-            const int k0 = t * kGemmBK;
+            const int k0 = (t_base + t) * kGemmBK;
             const uint32_t *wp = a.bvr + (static_cast<size_t>(k0 / 32 + bw) * N + n_ld) * S;
             // (ordinary loads: every row tile of the launch reads these again; non-temporal ones measured 2-3 % slower)
             const Planes<S> pl = load_planes<S>(wp);
@@ -1021,7 +1024,7 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
     }
     auto fetch_a = [&](int t) __attribute__((always_inline)) {        // tile t -> buffer t % 2, asynchronously
         unsigned char *dst = As + (t & 1) * kGemmATile + wave * 8192;
-        const uint16_t *src = a.x + static_cast<size_t>(t) * kGemmBK;
+        const uint16_t *src = a.x + static_cast<size_t>(t_base + t) * kGemmBK;
 #pragma unroll
         for (int j = 0; j < 8; ++j)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + xoff[j]),
@@ -1069,6 +1072,24 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
     }
 
     // ---- D[i][j] sits in lane j + 32*((i/4)%2), register (i%4) + 4*(i/8)
+    if (a.ksplit > 1) {
+        // K split across workgroups: every workgroup leaves its fp32 tile in `part`; sbvr_gemm_reduce_kernel,
+        // launched behind this kernel, adds the tiles up in the order of blockIdx.z and rounds once.
+        float *mine = a.part + blockIdx.z * (static_cast<size_t>(M) * N);
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj) {
+            const int n = n0 + wn * 64 + bj * 32 + (lane & 31);
+#pragma unroll
+            for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + wm * 128 + bi * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (m < M && n < N)
+                        mine[static_cast<size_t>(m) * N + n] = acc[bi][bj][r];
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj) {
         const int n = n0 + wn * 64 + bj * 32 + (lane & 31);
@@ -1088,6 +1109,36 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
                 }
             }
     }
+}
+
+// Second pass of a split prefill launch: out[m, n] = fp16(sum over z, in order, of part[z][m][n]) (+ bias),
+// and the partial results are set back to zero (the workspace is shared with the decode kernel's
+// accumulators, which must find zeros).  Four outputs per thread.
+__global__ void __launch_bounds__(256)
+sbvr_gemm_reduce_kernel(float *__restrict__ part, const uint16_t *__restrict__ bias, uint16_t *__restrict__ out,
+                        int M, int N, int ksplit)
+{
+    const size_t total = static_cast<size_t>(M) * N;
+    const size_t at = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+    if (at >= total)
+        return;
+    // (N is a multiple of 4 here, so the four outputs share a row and the 16-byte accesses are aligned)
+    v4f sum = {0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < ksplit; ++z) {
+        v4f *cell = reinterpret_cast<v4f *>(part + z * total + at);
+        sum += *cell;
+        *cell = v4f{0.f, 0.f, 0.f, 0.f};
+    }
+    const int n = static_cast<int>(at % N);
+    uint16_t r[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        r[i] = f2h(sum[i]);
+        if (bias)
+            r[i] = hadd(r[i], bias[n + i]);
+    }
+    *reinterpret_cast<uint2 *>(out + at) = uint2{static_cast<uint32_t>(r[0]) | (static_cast<uint32_t>(r[1]) << 16),
+                                                 static_cast<uint32_t>(r[2]) | (static_cast<uint32_t>(r[3]) << 16)};
 }
 
 // ------------------------------------------------- MFMA, 5 to 32 batch rows
@@ -1303,9 +1354,38 @@ bool gemm_path_ok(int M, int N, int K, int S, int G)
            static_cast<double>(K / 32) * N * S < 2147483648.0 && static_cast<double>(M) * K < 2147483648.0;
 }
 
+// Workgroups along K for the prefill kernel: as long as the output tiles alone leave half of the
+// chip's 256 CUs without a workgroup, and a part keeps at least 16 steps.  A function of the shape
+// only, so that the workspace can be sized without a device.
+constexpr int kGemmSplitCus = 256, kGemmMaxKsplit = 8;
+
+int gemm_tiles(int M, int N)
+{
+    return ((N + kGemmBN - 1) / kGemmBN) * ((M + kGemmBM - 1) / kGemmBM);
+}
+
+int gemm_ksplit(int M, int N, int K)
+{
+    const int tiles = gemm_tiles(M, N), steps = K / kGemmBK;
+    int ks = 1;
+    if (N % 4)                  // the second pass works on four outputs of a row at a time
+        return 1;
+    while (ks < kGemmMaxKsplit && tiles * ks * 2 <= kGemmSplitCus && steps % (ks * 2) == 0 && steps / (ks * 2) >= 16)
+        ks *= 2;
+    return ks;
+}
+
+// Workspace of the split prefill launch: the partial results.
+size_t gemm_workspace_bytes(int M, int N, int K)
+{
+    const int ks = gemm_ksplit(M, N, K);
+    return ks == 1 ? 0 : static_cast<size_t>(ks) * M * N * sizeof(float);
+}
+
 hipError_t launch_gemm(int S, const GemmArgs &a, hipStream_t st)
 {
-    const dim3 grid(static_cast<unsigned>((a.N + kGemmBN - 1) / kGemmBN), static_cast<unsigned>((a.M + kGemmBM - 1) / kGemmBM));
+    const dim3 grid(static_cast<unsigned>((a.N + kGemmBN - 1) / kGemmBN), static_cast<unsigned>((a.M + kGemmBM - 1) / kGemmBM),
+                    static_cast<unsigned>(a.ksplit));
     const dim3 block(kGemmThreads);
     const size_t lds = 2 * (kGemmATile + kGemmBTile);      // 96 KiB: above the 64 KiB a kernel gets without asking
 #define SBVR_GEMM_LAUNCH(SS)                                                                                   \
@@ -1730,9 +1810,11 @@ int sbvr_hip_init(int device)
 
 size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G)
 {
-    if (!mfma_path_ok(M, N, K, S, G))
-        return 0;
-    return static_cast<size_t>(M) * N * sizeof(unsigned long long);
+    if (mfma_path_ok(M, N, K, S, G))
+        return static_cast<size_t>(M) * N * sizeof(unsigned long long);
+    if (gemm_path_ok(M, N, K, S, G) && !rows32_path_ok(M, N, K, S, G))
+        return gemm_workspace_bytes(M, N, K);
+    return 0;
 }
 
 }  // extern "C"
@@ -1859,10 +1941,24 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         g.M = M; g.N = N; g.K = K; g.L = L;
         g.steps_per_group = G / kGemmBK;
         g.idx16 = idx_bytes == 2;
+        g.ksplit = 1;
+        // K split across workgroups where the output tiles alone would leave CUs idle, if the caller brought the
+        // workspace for it (without one the launch is simply not split)
+        const size_t need = gemm_workspace_bytes(M, N, K);
+        if (need && workspace && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+            g.ksplit = gemm_ksplit(M, N, K);
+            g.part = static_cast<float *>(workspace);
+        }
 #ifdef SBVR_TRACE
         g.trace = g_trace;
 #endif
-        const hipError_t e = launch_gemm(S, g, st);
+        hipError_t e = launch_gemm(S, g, st);
+        if (e == hipSuccess && g.ksplit > 1) {
+            const size_t quads = (static_cast<size_t>(M) * N + 3) / 4;
+            hipLaunchKernelGGL(sbvr_gemm_reduce_kernel, dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256), 0, st,
+                               g.part, g.bias, g.out, M, N, g.ksplit);
+            e = hipGetLastError();
+        }
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "gemm launch: %s", hipGetErrorString(e));
         return SBVR_HIP_OK;

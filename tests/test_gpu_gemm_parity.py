@@ -125,3 +125,51 @@ def test_linearity_70b_width():
     assert ((y12 - (y1 + y2)).abs() / torch.maximum(y12.abs(), rms)).max().item() < 4e-3
     row = sbvr._sbvr_linear_f16(x1[7:8].contiguous(), bvr, idx, cache, None, bvr_len=128).float()
     assert ((y1[7:8] - row).abs() / torch.maximum(row.abs(), rms)).max().item() < 4e-3
+
+
+@pytest.mark.parametrize("M,N,K,S,L,bias", [
+    (300, 512, 4096, 4, 256, False),       # 8 output tiles, K split 2 ways
+    (256, 384, 16384, 4, 300, True),       # 3 tiles, 8 ways, uint16 indices, bias
+    (520, 132, 8192, 3, 64, False),        # ragged M and N, 4 ways
+    (64, 1000, 2048, 2, 256, True),        # 2 ways at the smallest K that is split
+])
+def test_k_split_across_workgroups(oracle, M, N, K, S, L, bias):
+    """Few output tiles: the prefill launch splits K across workgroups through the caller's workspace.
+    Same tolerance as the unsplit launch, the same bits on a second call, and the workspace zero again."""
+    import sbvr
+    from sbvr import hip, synth
+    dev = torch.device("cuda:0")
+    lib = hip._load()
+    need = lib.sbvr_hip_linear_f16_workspace(M, N, K, S, 128)
+    assert need > M * N * 4, "this shape should ask for a split-K workspace"
+    run_case(oracle, N, K, S, 128, M, L, seed=K // 64 + M, bias=bias)
+    bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(N, K, S, 128, L, seed=1))
+    x = torch.randn((M, K), generator=torch.Generator().manual_seed(2)).to(torch.float16).to(dev)
+    a = sbvr._sbvr_linear_f16(x, bvr, idx, cache, bvr_len=128).clone()
+    b = sbvr._sbvr_linear_f16(x, bvr, idx, cache, bvr_len=128)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b), "split-K result depends on the order of arrival"
+    ws = hip._workspaces[(dev.index, torch.cuda.current_stream(dev).cuda_stream)]
+    assert ws.numel() >= need and int(ws.count_nonzero()) == 0, "workspace not left zero-filled"
+    # a decode launch that shares the workspace right after it
+    y1 = sbvr._sbvr_linear_f16(x[:1].contiguous(), bvr, idx, cache, bvr_len=128)
+    _, yd = oracle.C.linear_f16(x[:1].cpu().numpy(), bvr.cpu().numpy(), idx.cpu().numpy(), cache.cpu().numpy(), 128)
+    assert np.abs(y1.float().cpu().numpy() - yd).max() <= 1e-2 * max(np.abs(yd).max(), 1e-6)
+
+
+def test_k_split_without_workspace_is_not_split(oracle):
+    """Through the C ABI with no workspace the same shape runs unsplit and gives the unsplit result."""
+    import ctypes
+    from sbvr import hip, synth
+    dev = torch.device("cuda:0")
+    lib = hip._load()
+    M, N, K, S, L = 300, 512, 4096, 4, 256
+    bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(N, K, S, 128, L, seed=5))
+    x = torch.randn((M, K), generator=torch.Generator().manual_seed(6)).to(torch.float16).to(dev)
+    out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    rc = lib.sbvr_hip_linear_f16(x.data_ptr(), bvr.data_ptr(), idx.data_ptr(), 1, cache.data_ptr(), None, out.data_ptr(),
+                                 M, N, K, S, 128, L, None, 0, 0, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert rc == 0
+    _, yd = oracle.C.linear_f16(x.cpu().numpy(), bvr.cpu().numpy(), idx.cpu().numpy(), cache.cpu().numpy(), 128)
+    check(out, yd, "unsplit launch without a workspace")
