@@ -129,8 +129,8 @@ def test_linearity_70b_width():
 
 @pytest.mark.parametrize("M,N,K,S,L,bias", [
     (300, 512, 4096, 4, 256, False),       # 8 output tiles, K split 2 ways
-    (256, 384, 16384, 4, 300, True),       # 3 tiles, 8 ways, uint16 indices, bias
-    (520, 132, 8192, 3, 64, False),        # ragged M and N, 4 ways
+    (100, 128, 16384, 4, 300, True),       # 1 tile, 8 ways, uint16 indices, bias
+    (520, 132, 4096, 3, 64, False),        # ragged M and N
     (64, 1000, 2048, 2, 256, True),        # 2 ways at the smallest K that is split
 ])
 def test_k_split_across_workgroups(oracle, M, N, K, S, L, bias):
