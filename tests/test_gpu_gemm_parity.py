@@ -128,7 +128,7 @@ def test_linearity_70b_width():
 
 
 @pytest.mark.parametrize("M,N,K,S,L,bias", [
-    (300, 512, 4096, 4, 256, False),       # 8 output tiles, K split 2 ways
+    (300, 256, 4096, 4, 256, False),       # 4 output tiles, K split 2 ways
     (100, 128, 16384, 4, 300, True),       # 1 tile, 8 ways, uint16 indices, bias
     (520, 132, 4096, 3, 64, False),        # ragged M and N
     (64, 1000, 2048, 2, 256, True),        # 2 ways at the smallest K that is split
@@ -163,7 +163,7 @@ def test_k_split_without_workspace_is_not_split(oracle):
     from sbvr import hip, synth
     dev = torch.device("cuda:0")
     lib = hip._load()
-    M, N, K, S, L = 300, 512, 4096, 4, 256
+    M, N, K, S, L = 300, 256, 4096, 4, 256
     bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(N, K, S, 128, L, seed=5))
     x = torch.randn((M, K), generator=torch.Generator().manual_seed(6)).to(torch.float16).to(dev)
     out = torch.empty((M, N), dtype=torch.float16, device=dev)
