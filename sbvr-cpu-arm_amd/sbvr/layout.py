@@ -118,3 +118,33 @@ def rewidth(bvr, dtype):
         raise ValueError("byte count per row must be a multiple of 4")
     b = bvr.view(Kw // 4, 4, R, S).permute(0, 2, 3, 1).contiguous()
     return b.view(torch.uint32).view(Kw // 4, R, S)
+
+
+def fuse_rows(parts):
+    """One encoding of the row-wise concatenation of several encoded matrices.
+
+    ``parts``: (bvr (Kw, N_i, S), coeff_idx (Kg, N_i), coeff_cache (L_i, S)) in the
+    default layout, all with the same K, group length and plane count.  The
+    tables are concatenated and every part's indices are shifted by the lines in
+    front of it, so the result decodes to the parts' weights stacked on top of
+    each other: q|k|v or gate|up of models/sbvr_llama.py:239, 319-321 as one
+    operand (one launch instead of three or two).  Returns (bvr, coeff_idx, coeff_cache)."""
+    if not parts:
+        raise ValueError("nothing to fuse")
+    bvr0, idx0, cache0 = parts[0]
+    for bvr, idx, cache in parts:
+        if bvr.dim() != 3 or bvr.shape[0] != bvr0.shape[0] or bvr.shape[2] != bvr0.shape[2] or bvr.dtype != bvr0.dtype:
+            raise ValueError("parts must share K, the plane count and the word type")
+        if idx.shape[0] != idx0.shape[0] or idx.shape[1] != bvr.shape[1] or cache.shape[1] != bvr.shape[2]:
+            raise ValueError("parts must share the group length, and their arrays must fit together")
+    lines = sum(int(c.shape[0]) for _, _, c in parts)
+    if lines > 65536:
+        raise ValueError(f"{lines} coefficient lines do not fit 16-bit indices")
+    idx_dtype = torch.uint8 if lines <= 256 else torch.uint16
+    shifted, base = [], 0
+    for _, idx, cache in parts:
+        shifted.append((idx.to(torch.int32) + base).to(idx_dtype))
+        base += int(cache.shape[0])
+    return (torch.cat([b for b, _, _ in parts], dim=1).contiguous(),
+            torch.cat(shifted, dim=1).contiguous(),
+            torch.cat([c for _, _, c in parts], dim=0).contiguous())

@@ -4,7 +4,7 @@ intended forward is ``x @ restored_weight.T`` (:86-87); this one holds the three
 arrays of an ``sbvr`` object and calls the HIP operator."""
 import torch
 
-from . import hip
+from . import hip, layout
 
 
 class SBVRLinear(torch.nn.Module):
@@ -29,6 +29,21 @@ class SBVRLinear(torch.nn.Module):
         return cls(in_features, out_features, enc.default_layout(torch.uint32), enc.coeff_idx.data,
                    enc.coeff_cache.data, enc.bvr_len, bias)
 
+    @classmethod
+    def fused(cls, encs, biases=None):
+        """One layer for several ``sbvr`` objects that share their input (q, k, v or
+        gate, up): the weights stacked row-wise, see layout.fuse_rows.  The output
+        holds the parts' outputs side by side."""
+        if any(e.original_data_shape[1] != encs[0].original_data_shape[1] or e.bvr_len != encs[0].bvr_len for e in encs):
+            raise ValueError("fused layers must share in_features and the group length")
+        bvr, idx, cache = layout.fuse_rows([(e.default_layout(torch.uint32), e.coeff_idx.data, e.coeff_cache.data)
+                                            for e in encs])
+        bias = None
+        if biases is not None:
+            bias = torch.cat([b.to(torch.float16) for b in biases])
+        return cls(encs[0].original_data_shape[1], sum(e.original_data_shape[0] for e in encs), bvr, idx, cache,
+                   encs[0].bvr_len, bias)
+
     def forward(self, x):
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1])
@@ -37,13 +52,7 @@ class SBVRLinear(torch.nn.Module):
         if x2.shape[1] != self.k_padded:      # the encoder pads K to a multiple of bvr_len
             x2 = torch.nn.functional.pad(x2, (0, self.k_padded - x2.shape[1]))
         x2 = x2.contiguous()
-        rows = x2.shape[0]
-        if rows <= 16:
-            y = hip._sbvr_linear_f16(x2, self.bvr, self.coeff_idx, self.coeff_cache, self.bias, self.bvr_len)
-        else:
-            parts = [hip._sbvr_linear_f16(x2[i:i + 16].contiguous(), self.bvr, self.coeff_idx,
-                                          self.coeff_cache, self.bias, self.bvr_len)
-                     for i in range(0, rows, 16)]
-            y = torch.cat(parts, dim=0)
+        # any number of rows: the operator picks the decode, 32-row or prefill kernel
+        y = hip._sbvr_linear_f16(x2, self.bvr, self.coeff_idx, self.coeff_cache, self.bias, self.bvr_len)
         y = y[:, :self.out_features]
         return y.reshape(*lead, self.out_features)

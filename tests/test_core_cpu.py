@@ -196,3 +196,18 @@ def test_torch_extension_mirrors_the_reference_operators():
         ops._sbvr_linear_f16(x, bvr, idx, cache)
     with pytest.raises(RuntimeError, match="must be on a GPU"):
         ops._sbvr_mm_T(bvr, idx, cache, bvr, idx, cache, torch.zeros(0, dtype=torch.float16))
+
+
+def test_fuse_rows_decodes_to_the_stacked_weights(oracle):
+    """layout.fuse_rows: tables concatenated, indices shifted; index width follows the total line count."""
+    from sbvr import layout, synth
+    parts = [synth.random_encoding(rows, 256, 3, 128, lines, seed=rows) for rows, lines in ((32, 100), (16, 100), (48, 60))]
+    bvr, idx, cache = layout.fuse_rows(parts)
+    assert bvr.shape == (8, 96, 3) and idx.shape == (2, 96) and cache.shape == (260, 3) and idx.dtype == torch.uint16
+    whole = oracle.C.decode(bvr.numpy(), idx.numpy(), cache.numpy(), 128)
+    stacked = np.concatenate([oracle.C.decode(b.numpy(), i.numpy(), c.numpy(), 128) for b, i, c in parts], axis=0)
+    assert np.array_equal(whole, stacked)
+    small = layout.fuse_rows(parts[:2])
+    assert small[1].dtype == torch.uint8 and small[2].shape[0] == 200
+    with pytest.raises(ValueError):
+        layout.fuse_rows([parts[0], synth.random_encoding(16, 512, 3, 128, 10, seed=1)])
