@@ -866,6 +866,28 @@ struct GemmArgs {
 #endif
 };
 
+// The S fp16 coefficients of one table line as packed pairs, in as few load instructions as the
+// line's alignment allows (a line starts at a multiple of 2*S bytes; the table is 16-byte aligned).
+template <int S>
+__device__ __forceinline__ void load_line_coeffs(const uint16_t *cp, uint32_t (&cr)[(S + 1) / 2])
+{
+    if constexpr (S == 4) {
+        const v2u t = *reinterpret_cast<const v2u *>(cp);
+        cr[0] = t.x; cr[1] = t.y;
+    } else if constexpr (S == 8) {
+        const v4u t = *reinterpret_cast<const v4u *>(cp);
+        cr[0] = t.x; cr[1] = t.y; cr[2] = t.z; cr[3] = t.w;
+    } else if constexpr (S % 2 == 0) {
+#pragma unroll
+        for (int j = 0; j < S / 2; ++j)
+            cr[j] = reinterpret_cast<const uint32_t *>(cp)[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < (S + 1) / 2; ++j)
+            cr[j] = static_cast<uint32_t>(cp[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(cp[2 * j + 1]) << 16 : 0u);
+    }
+}
+
 #ifdef SBVR_TRACE
 #define SBVR_GSTAMP(step, slot)                                                                   \
     do {                                                                                          \
@@ -928,13 +950,7 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             for (int j = 0; j < S; ++j)
                 wr[j] = pl.w[j];
             const uint16_t *cp = a.cache + static_cast<size_t>(line_of(line[0])) * S;
-#pragma unroll
-            for (int j = 0; j < (S + 1) / 2; ++j) {
-                if (S % 2 == 0 || 2 * j + 1 < S)
-                    cr[j] = static_cast<uint32_t>(cp[2 * j]) | (static_cast<uint32_t>(cp[2 * j + 1]) << 16);
-                else
-                    cr[j] = cp[2 * j];
-            }
+            load_line_coeffs<S>(cp, cr);
             line[0] = line[1];
             line[1] = load_line(min(t + 2, steps - 1));
         };
@@ -1227,14 +1243,7 @@ sbvr_gemm_rows32_kernel(const RowsArgs a)
                 b.xa[i][1] = *reinterpret_cast<const v4u *>(xrow + 32 * w + 16);
             }
             const int ln = min(a.idx16 ? (line[i] & 0xff) | ((line[i] >> 8) & 0xff00) : line[i] & 0xff, a.L - 1);
-            const uint16_t *cp = a.cache + static_cast<size_t>(ln) * S;
-#pragma unroll
-            for (int q = 0; q < CW; ++q) {
-                if (S % 2 == 0 || 2 * q + 1 < S)
-                    b.c[i][q] = static_cast<uint32_t>(cp[2 * q]) | (static_cast<uint32_t>(cp[2 * q + 1]) << 16);
-                else
-                    b.c[i][q] = cp[2 * q];
-            }
+            load_line_coeffs<S>(a.cache + static_cast<size_t>(ln) * S, b.c[i]);
         }
     };
 
@@ -1514,10 +1523,7 @@ sbvr_row_deq_lanes_kernel(const uint16_t *__restrict__ x, const uint32_t *__rest
     };
     constexpr int CW = (S + 1) / 2;
     auto load_coeffs = [&](int raw, uint32_t (&c)[CW]) __attribute__((always_inline)) {
-        const uint16_t *cp = cache + static_cast<size_t>(line_of(raw)) * S;
-#pragma unroll
-        for (int j = 0; j < CW; ++j)
-            c[j] = static_cast<uint32_t>(cp[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(cp[2 * j + 1]) << 16 : 0u);
+        load_line_coeffs<S>(cache + static_cast<size_t>(line_of(raw)) * S, c);
     };
     const int last = steps - 1;
     // pipeline: raw index of step i+2, and words / coefficients / activation of step i+1
@@ -2034,7 +2040,8 @@ int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_co
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (idx_bytes == 1 && L > 256)
         return fail(SBVR_HIP_EINVAL, "uint8 indices cannot address L=%d lines", L);
-    if (M <= 65535 && (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) && reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0) {
+    if (M <= 65535 && (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) && reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(r_coeff_cache) % 16 == 0) {
         // lanes along K; as many waves as there are steps of 64 rows, up to kRowDeqWaves
         const int steps = (K + 63) / 64;
         const int waves = steps < kRowDeqWaves ? steps : kRowDeqWaves;
