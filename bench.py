@@ -32,8 +32,8 @@ N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH = 14336, 4096, 4, 128, 256, 1
 COPIES = 16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the gate GEMV, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# 256 MiB copy (profiles/sbvr_gemv_mfma_gate_4096x14336.txt): 30.44 MB read + 0.60 MB written.
-MEASURED_TRAFFIC_BYTES = 31.04e6
+# 256 MiB copy (profiles/sbvr_gemv_mfma_gate_4096x14336.txt): 29.99 MB read + 0.60 MB written.
+MEASURED_TRAFFIC_BYTES = 30.59e6
 
 
 def algorithmic_bytes(n, k, s, g, lines, m):
