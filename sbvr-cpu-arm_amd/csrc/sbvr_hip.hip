@@ -844,9 +844,10 @@ hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, int xm, hipS
 // A SIMD holds one consumer and two producers, so the decode (VALU) and the
 // MFMAs overlap.  Both tiles are double-buffered; one barrier per step.  Rows of the
 // LDS tiles are 128 bytes; 16-byte chunk c of row r is stored at chunk
-// c ^ (r & 7), which keeps the 16-byte operand reads of a quarter wave on
-// different banks.
+// c ^ ((r >> 1) & 7), which keeps the 16-byte operand reads of a quarter wave
+// (16 rows, two of them per 256-byte line of banks) on different banks.
 constexpr int kGemmBM = 256, kGemmBN = 128, kGemmBK = 64, kGemmThreads = 768;     // 4 consumer + 8 producer waves
+constexpr int kGemmABufs = 3;       // activation tiles in LDS: the one in use and the next two
 constexpr int kGemmATile = kGemmBM * kGemmBK * 2, kGemmBTile = kGemmBN * kGemmBK * 2;
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -909,7 +910,7 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
 {
     extern __shared__ __align__(16) unsigned char gsm[];
     unsigned char *const As = gsm;                       // 2 tiles
-    unsigned char *const Bs = gsm + 2 * kGemmATile;      // 2 tiles
+    unsigned char *const Bs = gsm + kGemmABufs * kGemmATile;      // 2 tiles
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -926,26 +927,34 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
         const int bn = pt & (kGemmBN - 1), bw = (pt >> 7) & 1, bh = pt >> 8;
         const int n_ld = min(n0 + bn, N - 1);
         const int b_dst = bn * 128;
-        const int sw = bn & 7, cb = bw * 4;
+        const int sw = (bn >> 1) & 7, cb = bw * 4;       // chunk swizzle of row bn, see the consumers
 
         constexpr int CW = (S + 1) / 2;
         uint32_t wreg0[S], wreg1[S], wreg2[S];           // three register sets, used in rotation
         uint32_t creg0[CW], creg1[CW], creg2[CW];
-        int line[2] = {0, 0};       // line index of the tile to be requested next, and of the one after
+        // The aligned 32-bit word that holds the line index of the tile a register set is filled with next:
+        // loaded when the set is requested, used three steps later by the same set's next request, and
+        // untouched in between (a move, or a byte load's zero extension, ends up at the top of the loop,
+        // where it makes the step wait for the youngest loads in flight).
+        uint32_t raw0 = 0, raw1 = 0, raw2 = 0;
 
         // (two byte loads whatever the index width: a branch between a 16-bit and an 8-bit load
         // inside the loop would make every later wait a wait for all loads)
-        auto load_line = [&](int t) __attribute__((always_inline)) -> int {
+        auto line_address = [&](int t) __attribute__((always_inline)) -> uintptr_t {
             const size_t at = (static_cast<size_t>((t_base + t) / a.steps_per_group) * N + n_ld) << a.idx16;
-            const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
-            const int lo = ib[at], hi = ib[at + a.idx16];
-            return lo | (hi << 16);          // raw bytes: put together where the index is used, not here,
-        };                                   // or the wait for this youngest load would drain all loads
-        auto line_of = [&](int raw) __attribute__((always_inline)) -> int {
-            return min(a.idx16 ? (raw & 0xff) | ((raw >> 8) & 0xff00) : raw & 0xff, a.L - 1);
+            return reinterpret_cast<uintptr_t>(static_cast<const uint8_t *>(a.idx) + at);
+        };
+        auto load_line = [&](int t, uint32_t &raw) __attribute__((always_inline)) {
+            // (a global-memory pointer by type: from a bare integer the compiler would make a flat load,
+            // whose completion order it does not know)
+            raw = *reinterpret_cast<const __attribute__((address_space(1))) uint32_t *>(line_address(t) & ~static_cast<uintptr_t>(3));
+        };
+        auto line_of = [&](int t, uint32_t raw) __attribute__((always_inline)) -> int {
+            const uint32_t v = raw >> (8 * static_cast<uint32_t>(line_address(t) & 3));
+            return min(static_cast<int>(a.idx16 ? v & 0xffffu : v & 0xffu), a.L - 1);
         };
         // global loads of tile t into one register set
-        auto request = [&](int t, uint32_t (&wr)[S], uint32_t (&cr)[CW]) __attribute__((always_inline)) {
+        auto request = [&](int t, uint32_t (&wr)[S], uint32_t (&cr)[CW], uint32_t &raw) __attribute__((always_inline)) {
             const int k0 = (t_base + t) * kGemmBK;
             const uint32_t *wp = a.bvr + (static_cast<size_t>(k0 / 32 + bw) * N + n_ld) * S;
             // (ordinary loads: every row tile of the launch reads these again; non-temporal ones measured 2-3 % slower)
@@ -953,13 +962,24 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
 #pragma unroll
             for (int j = 0; j < S; ++j)
                 wr[j] = pl.w[j];
-            const uint16_t *cp = a.cache + static_cast<size_t>(line_of(line[0])) * S;
+            asm volatile("" : "+v"(raw));                // not to be taken apart before this step (see pin)
+            const uint16_t *cp = a.cache + static_cast<size_t>(line_of(t, raw)) * S;
             load_line_coeffs<S>(cp, cr);
-            line[0] = line[1];
-            line[1] = load_line(min(t + 2, steps - 1));
+            load_line(min(t + 3, steps - 1), raw);
+        };
+        // Makes a register set opaque at the start of the step that decodes it: without this the compiler
+        // moves part of the decode up into the step before (arithmetic may cross a barrier), where the
+        // set's loads are the youngest in flight and the wait for them drains the whole queue.
+        auto pin = [&](uint32_t (&wr)[S], uint32_t (&cr)[CW], uint32_t &) __attribute__((always_inline)) {
+#pragma unroll
+            for (int j = 0; j < S; ++j)
+                asm volatile("" : "+v"(wr[j]));
+#pragma unroll
+            for (int j = 0; j < CW; ++j)
+                asm volatile("" : "+v"(cr[j]));
         };
         // one register set -> LDS buffers t % 2
-        auto produce = [&](int t, const uint32_t (&wr)[S], const uint32_t (&cr)[CW]) __attribute__((always_inline)) {
+        auto produce = [&](int t, const uint32_t (&wr)[S], const uint32_t (&cr)[CW], uint32_t) __attribute__((always_inline)) {
             unsigned char *Bt = Bs + (t & 1) * kGemmBTile;
             uint32_t cbits[S];
 #pragma unroll
@@ -986,13 +1006,14 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             *reinterpret_cast<v4u *>(Bt + b_dst + (((cb + bh) ^ sw) << 4)) = lo;
             *reinterpret_cast<v4u *>(Bt + b_dst + (((cb + 2 + bh) ^ sw) << 4)) = hi;
         };
-#define SBVR_SET(n) wreg##n, creg##n
+#define SBVR_SET(n) wreg##n, creg##n, raw##n
         // Requests are never conditional (beyond the last tile they repeat it): after a
         // branch that may or may not have issued loads, the wait for an older set would
         // have to assume it had not, and wait for everything.
         const int last = steps - 1;
-        line[0] = load_line(0);
-        line[1] = load_line(min(1, last));
+        load_line(0, raw0);
+        load_line(min(1, last), raw1);
+        load_line(min(2, last), raw2);
         request(0, SBVR_SET(0));
         request(min(1, last), SBVR_SET(1));
         request(min(2, last), SBVR_SET(2));
@@ -1004,18 +1025,21 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             // (tiles beyond the last are produced too, from repeated loads, into buffers nobody reads:
             // a loop body without branches keeps the waits of the three register sets apart)
             if (wave == 4) SBVR_GSTAMP(i, 2);
+            pin(SBVR_SET(1));
             request(min(i + 3, last), SBVR_SET(0));
             if (wave == 4) SBVR_GSTAMP(i, 3);
             produce(i + 1, SBVR_SET(1));
             if (wave == 4) SBVR_GSTAMP(i, 4);
             __syncthreads();
             if (wave == 4) SBVR_GSTAMP(i + 1, 2);
+            pin(SBVR_SET(2));
             request(min(i + 4, last), SBVR_SET(1));
             if (wave == 4) SBVR_GSTAMP(i + 1, 3);
             produce(i + 2, SBVR_SET(2));
             if (wave == 4) SBVR_GSTAMP(i + 1, 4);
             __syncthreads();
             if (wave == 4) SBVR_GSTAMP(i + 2, 2);
+            pin(SBVR_SET(0));
             request(min(i + 5, last), SBVR_SET(2));
             if (wave == 4) SBVR_GSTAMP(i + 2, 3);
             produce(i + 3, SBVR_SET(0));
@@ -1036,27 +1060,37 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             for (int r = 0; r < 16; ++r)
                 acc[bi][bj][r] = 0.f;
     const int wm = wave >> 1, wn = wave & 1;
-    const int arow = wm * 128 + (lane & 31), brow = wn * 64 + (lane & 31);      // + 32 bi / bj: same row & 7
-    const int rsw = lane & 7, chi = lane >> 5;
+    const int arow = wm * 128 + (lane & 31), brow = wn * 64 + (lane & 31);      // + 32 bi / bj: same (row >> 1) & 7
+    // Chunk c of tile row r sits at chunk position c ^ ((r >> 1) & 7) of the row's 128 bytes.  A 16-byte read
+    // is served 16 lanes (rows) at a time by 64 banks of 4 bytes, i.e. two rows side by side: with the row pair
+    // as the swizzle key the 16 rows hit 16 different bank groups (keyed by r & 7, rows r and r + 8 collided
+    // and every read took two turns).
+    const int rsw = (lane >> 1) & 7, chi = lane >> 5;
     // The activation tile goes from global memory straight into LDS (no registers): instruction j
     // of wave w fills the 1 KiB block 8w + j, i.e. rows 8 (8w + j) .. + 7, lane l the 16-byte slot l
-    // of it; with the row swizzle, slot l of a block holds chunk (l & 7) ^ (l >> 3) of row l >> 3.
+    // of it; with the row swizzle, slot l of a block holds chunk (l & 7) ^ ((4j + (l >> 4)) & 7) of row l >> 3.
     uint32_t xoff[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int row = 8 * (8 * wave + j) + (lane >> 3);
-        xoff[j] = static_cast<uint32_t>(min(m0 + row, M - 1)) * K + 8 * ((lane & 7) ^ (lane >> 3));     // M * K < 2^31 (checked)
+        xoff[j] = static_cast<uint32_t>(min(m0 + row, M - 1)) * K + 8 * ((lane & 7) ^ ((row >> 1) & 7));     // M * K < 2^31 (checked)
     }
-    auto fetch_a = [&](int t) __attribute__((always_inline)) {        // tile t -> buffer t % 2, asynchronously
-        unsigned char *dst = As + (t & 1) * kGemmATile + wave * 8192;
+    auto fetch_a = [&](int t, int buf) __attribute__((always_inline)) {        // tile t -> buffer buf, asynchronously
+        unsigned char *dst = As + buf * kGemmATile + wave * 8192;
         const uint16_t *src = a.x + static_cast<size_t>(t_base + t) * kGemmBK;
+        // Written as assembly (M0 = LDS address of lane 0's slot): the compiler counts the builtin form as a
+        // memory operation whose order of completion it does not know, and from then on turns every wait for
+        // an LDS read into a wait for all of them.
+        const uint32_t lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst));
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + xoff[j]),
-                                             (__attribute__((address_space(3))) void *)(dst + j * 1024), 16, 0, 0);
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         :: "v"(src + xoff[j]), "s"(lds + j * 1024) : "memory", "m0");
     };
-    fetch_a(0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): the tile is in LDS
+    fetch_a(0, 0);
+    fetch_a(min(1, steps - 1), 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): the tiles are in LDS
+    int cur = 0;                                 // activation buffer of tile i
     __syncthreads();
     // operand registers of two k-slices in turn: the reads of slice s+1 are issued before the MFMAs of slice s
     auto read_slice = [&](const unsigned char *At, const unsigned char *Bt, int ks, v8h (&af)[4], v8h (&bf)[2])
@@ -1078,9 +1112,13 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
     };
     for (int i = 0; i < 3 * rounds; ++i) {
         if (i < steps) {
-            const unsigned char *At = As + (i & 1) * kGemmATile, *Bt = Bs + (i & 1) * kGemmBTile;
+            const unsigned char *At = As + cur * kGemmATile, *Bt = Bs + (i & 1) * kGemmBTile;
             if (wave == 0) SBVR_GSTAMP(i, 0);
-            fetch_a(min(i + 1, steps - 1));      // lands in the other buffer while this one is used
+            // the tile after the next goes to the buffer that the tile before this one has left; it has two
+            // steps to land
+            fetch_a(min(i + 2, steps - 1), cur == 0 ? 2 : cur - 1);
+            // (With 168 registers a wave the compiler keeps one activation operand at a time and moves each
+            // read down to its MFMAs: fenced into the order written here the loop needs about 200.)
             v8h af0[4], bf0[2], af1[4], bf1[2];
             read_slice(At, Bt, 0, af0, bf0);
             read_slice(At, Bt, 1, af1, bf1);
@@ -1091,10 +1129,14 @@ sbvr_gemm_mfma_kernel(const GemmArgs a)
             mfma_slice(af0, bf0);
             mfma_slice(af1, bf1);
             if (wave == 0) SBVR_GSTAMP(i, 1);
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the next tile is in LDS
+            __builtin_amdgcn_sched_barrier(0);   // (or the wait moves up in front of the MFMAs)
+            __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8): all but the 8 loads above, i.e. this wave's part of the next tile is in LDS
+            cur = cur == 2 ? 0 : cur + 1;
         }
         __syncthreads();
     }
+
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // no load into LDS is left in flight when the wave ends
 
     // ---- D[i][j] sits in lane j + 32*((i/4)%2), register (i%4) + 4*(i/8)
     if (a.ksplit > 1) {
@@ -1405,7 +1447,7 @@ hipError_t launch_gemm(int S, const GemmArgs &a, hipStream_t st)
     const dim3 grid(static_cast<unsigned>((a.N + kGemmBN - 1) / kGemmBN), static_cast<unsigned>((a.M + kGemmBM - 1) / kGemmBM),
                     static_cast<unsigned>(a.ksplit));
     const dim3 block(kGemmThreads);
-    const size_t lds = 2 * (kGemmATile + kGemmBTile);      // 96 KiB: above the 64 KiB a kernel gets without asking
+    const size_t lds = kGemmABufs * kGemmATile + 2 * kGemmBTile;      // 128 KiB: above the 64 KiB a kernel gets without asking
 #define SBVR_GEMM_LAUNCH(SS)                                                                                   \
     {                                                                                                          \
         static bool raised_on[16] = {};                                                                        \
