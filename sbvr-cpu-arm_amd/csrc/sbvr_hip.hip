@@ -839,10 +839,11 @@ hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, int xm, hipS
 //     consumers, in three register sets used in rotation;
 //   * waves 0-3 run v_mfma_f32_32x32x16_f16 over the two tiles (each wave
 //     128 x 64 of the output, 8 accumulator blocks) and, before that, send for
-//     the 256 x 64 activations of the next step: global memory to LDS directly,
+//     the 256 x 64 activations of the step after the next: global memory to LDS directly,
 //     no registers, the data lands while the MFMAs run.
 // A SIMD holds one consumer and two producers, so the decode (VALU) and the
-// MFMAs overlap.  Both tiles are double-buffered; one barrier per step.  Rows of the
+// MFMAs overlap.  The weight tile has two buffers, the activation tile three (its
+// loads go out two steps ahead); one barrier per step.  Rows of the
 // LDS tiles are 128 bytes; 16-byte chunk c of row r is stored at chunk
 // c ^ ((r >> 1) & 7), which keeps the 16-byte operand reads of a quarter wave
 // (16 rows, two of them per 256-byte line of banks) on different banks.
