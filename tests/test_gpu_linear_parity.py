@@ -96,6 +96,30 @@ def test_sweep_gate(oracle, S, M):
     run_case(oracle, 14336, 4096, S, 128, M, 256, seed=12, flags=2 if M > 4 else 0)
 
 
+@pytest.mark.parametrize("S", [2, 3, 4])
+@pytest.mark.parametrize("M", [4, 8])
+def test_sweep_down(oracle, S, M):
+    """The other shape of the batch / plane sweep: 14336 -> 4096, long K (split across workgroups)."""
+    run_case(oracle, 4096, 14336, S, 128, M, 256, seed=14, flags=2 if M > 4 else 0)
+
+
+def test_sweep_down_default_path_16_rows(oracle):
+    """16 rows at the down shape without flags: whatever kernel the operator picks, same tolerance."""
+    import sbvr
+    from sbvr import synth
+    dev = _dev()
+    N, K, S, M = 4096, 14336, 4, 16
+    bvr, idx, cache = synth.random_encoding(N, K, S, 128, 256, seed=15)
+    x = torch.randn((M, K), generator=torch.Generator().manual_seed(16)).to(torch.float16)
+    y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev), None, bvr_len=128)
+    _, yd = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), 128)
+    got = y.float().cpu().numpy().astype(np.float64)
+    rms = float(np.sqrt(np.mean(yd ** 2)))
+    # (the 32-row kernel decodes the weights to fp16 first: judged against half the RMS for small outputs,
+    # as in test_gpu_gemm_parity.py)
+    assert (np.abs(got - yd) / np.maximum(np.abs(yd), 0.5 * rms)).max() <= 1e-2
+
+
 def test_portable_kernel(oracle):
     run_case(oracle, 100, 512, 4, 128, 1, 256, seed=13, flags=1)
     run_case(oracle, 96, 320, 5, 64, 3, 40, seed=14)       # no MFMA kernel for G=64 / S=5
