@@ -58,6 +58,13 @@ def test_ragged_n(oracle, N):
     run_case(oracle, N, 256, 4, 128, 33, 64, seed=30 + N)
 
 
+@pytest.mark.parametrize("K,G", [(64, 64), (128, 64), (128, 128), (192, 64), (256, 256)])
+def test_fewer_steps_than_pipeline_stages(oracle, K, G):
+    """1 to 4 steps of 64 along K: shorter than the three-step rotation of the weight loads and the
+    two-step lead of the activation loads."""
+    run_case(oracle, 200, K, 4, G, 70, 100, seed=60 + K + G)
+
+
 def test_u16_index_and_bias(oracle):
     run_case(oracle, 320, 768, 4, 128, 50, 3000, seed=41)
     run_case(oracle, 320, 768, 3, 128, 50, 256, seed=42, bias=True)
