@@ -113,6 +113,19 @@ int sbvr_hip_linear_f16_add_rmsnorm(const void *x, const void *delta, const void
                                     void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: the launch that
+ * sbvr_hip_linear_f16 would make for one row of this shape (same grid, same
+ * workgroups, the same plane-word and line-index requests in the same order)
+ * with everything else left out: no activations, no arithmetic, nothing
+ * written to out.  Its duration is what the memory system alone needs for the
+ * weight stream of that launch; bench.py --stream-floor times it beside the
+ * real kernel.  Same shape limits as the fused one-row linears above.
+ */
+int sbvr_hip_linear_f16_stream_floor(const uint32_t *bvr, const void *coeff_idx, int idx_bytes,
+                                     const void *coeff_cache, void *out, int N, int K, int S, int G, int L,
+                                     void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * fp16 activations against a weight encoded with trans=True (groups along N):
  *   r_bvr (N/32, K, S) uint32, r_coeff_idx (N/G, K), r_coeff_cache (L, S) fp16
  *   out[m,n] = f16( bias[n] + sum_k x[m,k] * sum_j c[idx[n/G,k], j] * bit_j )

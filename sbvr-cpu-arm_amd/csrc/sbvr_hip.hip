@@ -39,6 +39,7 @@
 //
 // Portable kernels (any shape, one thread per output) back all of them.
 #include <hip/hip_runtime.h>
+#include <mutex>
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -140,6 +141,7 @@ sbvr_linear_portable_kernel(const uint16_t *__restrict__ x, const uint32_t *__re
 constexpr int kSub = 128;        // K elements per MFMA (one sub-group)
 constexpr int kMaxWaves = 16;    // waves of a workgroup; they split K among themselves
 constexpr int kMaxM = 16;        // batch rows of the decode kernel (row tiles of 4)
+constexpr int kUnitsAhead = 3;   // units of plane words a wave of the decode kernel keeps in flight
 constexpr float kLastTermScale = 256.f;  // third fp8 term of an activation holds residual * 256
 
 // Split-K accumulator: one 64-bit word per output, [count:8 | sum:56].  Every
@@ -164,6 +166,7 @@ struct GemvArgs {
     int idx16;            // line indices are uint16 (else uint8)
     int ksplit;           // workgroups along K
     int xstride;          // elements between batch rows of x
+    int wstride;          // columns a workgroup owns: a multiple of 8, (CT - 1) * 16 < wstride <= CT * 16
     // fused activation prologues (see XM of the kernel)
     const uint16_t *delta;      // XM == 2: added to x before the norm
     const uint16_t *norm_w;     // XM == 2: RMSNorm weight
@@ -177,8 +180,8 @@ struct GemvArgs {
 #ifdef SBVR_TRACE
 #define SBVR_STAMP(i)                                                         \
     do {                                                                      \
-        if (a.trace && threadIdx.x == 0)                                      \
-            a.trace[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = wall_clock64();                   \
+        if (a.trace && (threadIdx.x & 63) == 0)                               \
+            a.trace[((blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64(); \
     } while (0)
 unsigned long long *g_trace = nullptr;
 #else
@@ -292,6 +295,7 @@ __device__ __forceinline__ float wave_fsum(float v)
 //             where the waves then find their own elements; workgroup (0, 0) writes r
 //             to x_out.
 constexpr int kXPlain = 0, kXSwiGLU = 1, kXAddNorm = 2, kXAddNorm2 = 3;   // (3: two chunks of x per thread for the norm)
+constexpr int kXFloor = 4;      // measurement aid: the launch's plane-word and index requests only, no arithmetic, no output
 constexpr int kNormChunksMax = 2;             // 16-byte chunks of x a thread sums for the norm, at most
 
 __device__ __forceinline__ uint32_t swiglu_pair(uint32_t g, uint32_t u)
@@ -336,8 +340,9 @@ __device__ __forceinline__ long long to_fixed(float y)
 // of plane words.  The waves share nothing until their partial results meet in
 // LDS, so nothing in a wave waits for another wave before that.  Straight-line
 // code; every wait is for exactly the oldest outstanding load.  In a wave:
-//   1. all its requests at once: its activations (one dword per lane, row and
-//      sub-group), the line indices of its units, the plane words;
+//   1. its first requests: its activations (one dword per lane, row and
+//      sub-group), the line indices of its units, the plane words of its first
+//      units (the later units are requested one at a time, in step 4);
 //   2. the activations arrive first: they become the fp8 A operands (through
 //      a 2 KiB LDS buffer of the wave's own, which does the byte transpose);
 //   3. the indices arrive: the coefficient lines are gathered (vector loads
@@ -360,15 +365,21 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     const int col = lane & 15;   // column inside a tile (B and D operands)
     const int blk = lane >> 4;   // word of the sub-group (B), batch row of the tile (D)
     const int sg0 = (blockIdx.y * waves + wave) * SP;     // first sub-group of this wave
-    // The workgroup owns columns [n_own, n_own + 16*CT).  It computes a full
-    // window of 16*CT columns; a window that would stick out of N is moved left,
-    // and the columns it then shares with its neighbour are left to the neighbour.
+    // The workgroup owns columns [n_own, n_own + wstride), wstride <= 16*CT a multiple
+    // of 8 (half a tile is 128 bytes per word of K: whole cache lines).  It computes
+    // a full window of 16*CT columns; a window that would stick out of N is moved
+    // left, and the columns it then shares with its neighbour are left to the
+    // neighbour.
     // Workgroups go to the 8 XCDs in turn (by their linear index, x first): give each XCD a contiguous range of
     // column windows instead of every eighth one (2-3 % at the 4096 <-> 14336 shapes).
     const int bx = gridDim.x % 8 == 0 ? static_cast<int>((blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8)
                                       : static_cast<int>(blockIdx.x);
-    const int n_own = bx * CT * 16;
+    const int n_own = bx * a.wstride;
     const int n_base = min(n_own, N - CT * 16);
+    // columns of the window that are this workgroup's to load: with wstride < 16*CT the rest of the last
+    // tile is the next workgroup's (those lanes repeat the last own column: same cache line, no traffic,
+    // and their results are dropped); a window moved left at the edge of N loads all of its columns
+    const int w_lim = n_base == n_own ? a.wstride : CT * 16;
     unsigned char *const mine = smem + wave * 2048;        // this wave's buffer
 
     SBVR_STAMP(0);
@@ -380,7 +391,9 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     uint32_t x2[XM == kXSwiGLU ? SP : 1][XM == kXSwiGLU ? MT : 1][4];   // up (SwiGLU)
     uint32_t xw[kNorm ? SP : 1];                                        // norm weights
     v4u sx[NV], sd[NV];                                                 // this thread's share of all of x and delta
-    if constexpr (!kNorm) {
+    if constexpr (XM == kXFloor) {
+        // (no activations)
+    } else if constexpr (!kNorm) {
 #pragma unroll
         for (int sgi = 0; sgi < SP; ++sgi)
 #pragma unroll
@@ -426,15 +439,40 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
         }
     }
     Planes<S> q[U];
-    {
-        const uint32_t lane_w = (static_cast<uint32_t>(blk) * N + n_base + col) * S;   // words
+    const uint32_t lane_w = (static_cast<uint32_t>(blk) * N + n_base + col) * S;   // words
+    const uint32_t lane_w_last = (static_cast<uint32_t>(blk) * N + n_base + min((CT - 1) * 16 + col, w_lim - 1)) * S;
+    auto request_units = [&](int u0, int u1) __attribute__((always_inline)) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const uint32_t *wrow = a.bvr + static_cast<size_t>(sg0 + u / CT) * 4 * N * S;     // wave-uniform
-            q[u] = load_planes<S, true>(wrow + lane_w + (u % CT) * 16 * S);
-        }
+        for (int u = 0; u < U; ++u)
+            if (u >= u0 && u < u1) {
+                const uint32_t *wrow = a.bvr + static_cast<size_t>(sg0 + u / CT) * 4 * N * S;     // wave-uniform
+                q[u] = load_planes<S, true>(u % CT == CT - 1 ? wrow + lane_w_last : wrow + lane_w + (u % CT) * 16 * S);
+            }
+    };
+    if constexpr (XM == kXFloor) {
+        // every request of the real launch, then nothing: how long the memory system alone takes
+        request_units(0, U);
+        uint32_t seen = 0;
+#pragma unroll
+        for (int sgi = 0; sgi < SP; ++sgi)
+            seen ^= static_cast<uint32_t>(lraw[sgi]);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < S; ++j)
+                seen ^= q[u].w[j];
+        if (seen == 0x9e3779b9u && a.M == 0x7fffffff)       // never true: keeps the loads alive
+            a.out[lane] = static_cast<uint16_t>(seen);
+        return;
     }
-    __builtin_amdgcn_sched_barrier(0);       // every request is out before anything waits
+    // A wave keeps kUnitsAhead units in flight: the first ones are requested here, before the A operands are
+    // made, and each unit that is worked on asks for the one kUnitsAhead behind it.  A CU takes about 48 such
+    // requests at a time and hands the free places to its oldest waves first: a wave that asked for all of its
+    // units at once would sit in the issue of its loads for microseconds (the youngest waves until the launch
+    // is nearly over) and make its operands only after that.
+    constexpr int kPre = U < kUnitsAhead ? U : kUnitsAhead;
+    request_units(0, kPre);
+    __builtin_amdgcn_sched_barrier(0);       // these requests are out before anything waits
     SBVR_STAMP(1);
 
     // -- 2. A operands.  Lane l turns elements 2l and 2l+1 of a batch row into
@@ -480,18 +518,30 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
             xx[sgi][0][0] = reinterpret_cast<const uint32_t *>(rbuf)[(sg0 + sgi) * (kSub / 2) + lane];
         }
     }
+#ifdef SBVR_TRACE
+    if constexpr (!kNorm) {
+        asm volatile("" :: "v"(xx[SP - 1][0][0]));
+        SBVR_STAMP(7);
+    }
+#endif
+    // (raised priority: the SIMD's other waves are in their units by now, and this wave would get a turn
+    // only between their MFMAs -- measured up to 2.5 us for the 0.3 us of work; its own units wait for this)
+    __builtin_amdgcn_s_setprio(3);
     v8i A[SP][MT];
     float scale[SP][MT];         // of this lane's batch row (blk)
     const int m_rows = XM != kXPlain ? 1 : a.M;
-    {
-        const int off0 = a_image_byte_offset(2 * lane, 0), off1 = a_image_byte_offset(2 * lane + 1, 0);
-        const float fac0 = (lane & 1) ? 1.f : 4.f, fac1 = (lane & 1) ? 1.f : 2.f;
-        reinterpret_cast<uint4 *>(mine)[lane * 2] = uint4{0u, 0u, 0u, 0u};
-        reinterpret_cast<uint4 *>(mine)[lane * 2 + 1] = uint4{0u, 0u, 0u, 0u};
+    const int off0 = a_image_byte_offset(2 * lane, 0), off1 = a_image_byte_offset(2 * lane + 1, 0);
+    const float fac0 = (lane & 1) ? 1.f : 4.f, fac1 = (lane & 1) ? 1.f : 2.f;
+    // the operands of sub-groups [s0, s1) of this wave
+    auto make_operands = [&](int s0, int s1) __attribute__((always_inline)) {
 #pragma unroll
-        for (int mt = MT - 1; mt >= 0; --mt)
+        for (int sgi = 0; sgi < SP; ++sgi) {
+            if (sgi < s0 || sgi >= s1)
+                continue;
+            reinterpret_cast<uint4 *>(mine)[lane * 2] = uint4{0u, 0u, 0u, 0u};
+            reinterpret_cast<uint4 *>(mine)[lane * 2 + 1] = uint4{0u, 0u, 0u, 0u};
 #pragma unroll
-            for (int sgi = 0; sgi < SP; ++sgi) {
+            for (int mt = MT - 1; mt >= 0; --mt) {
                 scale[sgi][mt] = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -529,7 +579,10 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
                 }
                 A[sgi][mt] = *reinterpret_cast<const v8i *>(mine + lane * 32);
             }
-    }
+        }
+    };
+    make_operands(0, SP);
+    __builtin_amdgcn_s_setprio(0);
     SBVR_STAMP(2);
 
     // -- 3. coefficient lines (S fp16 each): lane l gathers the line of column n_base + l for each
@@ -563,6 +616,8 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int sgi = u / CT;
+        request_units(u + kPre, u + kPre + 1);      // keeps kPre units of this wave in flight
+        __builtin_amdgcn_sched_barrier(0);
         v4f D[MT][S];
 #pragma unroll
         for (int j = 0; j < S; ++j) {
@@ -639,7 +694,7 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
         for (int w = 0; w < waves; ++w)
             total += red[w * kRedStride + o * 64 + lane];
         const int n = n_base + ct * 16 + col, m = mt * 4 + blk;
-        const bool valid = m < a.M && (!shifted || n >= n_own);
+        const bool valid = m < a.M && (!shifted || n >= n_own) && n < n_own + a.wstride;
         const size_t at = static_cast<size_t>(m) * N + n;
         if (a.ksplit > 1) {
             // through the accumulators: the adder that completes the count converts
@@ -682,12 +737,25 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 struct GemvPlan {
     int CT, SP, MT, waves, n_wgs, ksplit;
     size_t lds;
+    int wstride;
 };
 
-int env_int(const char *name, int dflt)
+// Development switches, read from the environment once per process.
+struct EnvSwitches {
+    int ct, sp, waves, wstride, show_plan, popc_q;
+};
+
+const EnvSwitches &env_switches()
 {
-    const char *v = getenv(name);
-    return v && *v ? atoi(v) : dflt;
+    static const EnvSwitches e = [] {
+        auto get = [](const char *name) {
+            const char *v = getenv(name);
+            return v && *v ? atoi(v) : 0;
+        };
+        return EnvSwitches{get("SBVR_HIP_CT"), get("SBVR_HIP_SP"), get("SBVR_HIP_WAVES"), get("SBVR_HIP_WSTRIDE"),
+                           get("SBVR_HIP_SHOW_PLAN"), get("SBVR_HIP_POPC_Q")};
+    }();
+    return e;
 }
 
 // (CT, SP) pairs that have a kernel instance; see the dispatch below.
@@ -703,61 +771,120 @@ bool shape_ok_for(int MT, int CT, int SP)
     return CT * MT <= 16 && (MT == 1 || CT * SP * MT <= 16);
 }
 
-// Picks the launch shape.  Measured on MI355X (Llama-3-8B layer shapes, batch 1),
-// all sensible shapes are within a few percent of each other once these hold:
-//  - about 4 units per wave when there is enough work for 2048 such waves,
+bool has_instance(int CT, int SP)
+{
+    for (int i = 0; i < kNumShapes; ++i)
+        if (kShapes[i][0] == CT && kShapes[i][1] == SP)
+            return true;
+    return false;
+}
+
+// Picks the launch shape.  Measured on MI355X (Llama-3-8B layer shapes, batch 1):
+//  1. Where 16 waves can cover all of K with at most two sub-groups per column tile each, one workgroup
+//     takes all of K (no accumulators, no atomics) and the columns are cut into windows of a multiple of
+//     8 columns such that the workgroups are a whole multiple of the CUs: the launch is bound by what a CU
+//     can have in flight, so a CU with 4 workgroups where others have 3 sets the time of the whole launch
+//     (4096 -> 14336 on 256 CUs: 256 windows of 56 columns, 7.9 us against 8.6 us for 224 x 4 of 64).
+//  2. Otherwise:
+//  - about 4 units per wave when there is enough work for 2048 such waves, 8 with four times that,
 //    fewer otherwise, with as many of them as possible along N (one sub-group
 //    per wave means one set of A operands per wave);
 //  - at least two workgroups per CU, so K is split across workgroups (through
 //    the accumulators) when N alone does not give that many;
 //  - the largest workgroup that keeps that, but no more than 8 waves when the
 //    waves do not all fit on the chip at once (finer placement).
-GemvPlan plan_gemv(int M, int N, int K, int S, int cus, int min_waves = 1)
+GemvPlan plan_gemv_uncached(int M, int N, int K, int S, int cus, int min_waves)
 {
     const int nsub = K / kSub;
     const int MT = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
     const int tiles16 = (N + 15) / 16;
-    const int eCT = env_int("SBVR_HIP_CT", 0), eSP = env_int("SBVR_HIP_SP", 0), eW = env_int("SBVR_HIP_WAVES", 0);
-    const long units = static_cast<long>(tiles16) * nsub;
-    int want = units >= 4L * 2048 ? 4 : (units >= 2L * 2048 ? 2 : 1);
-    while (want > 1 && !shape_ok_for(MT, want, 1))
-        want /= 2;
+    const EnvSwitches &env = env_switches();
+    const int eCT = env.ct, eSP = env.sp, eW = env.waves;
     GemvPlan best{};
-    double best_cost = 1e30;
-    for (int i = 0; i < kNumShapes; ++i) {
-        const int CT = kShapes[i][0], SP = kShapes[i][1];
-        if (nsub % SP || !shape_ok_for(MT, CT, SP) || CT * 16 > N)
-            continue;
-        if (eCT > 0 && eSP > 0 && (CT != eCT || SP != eSP))
-            continue;
-        const int parts = nsub / SP;             // wave-sized pieces of K
-        const int n_wgs = (tiles16 + CT - 1) / CT;
-        const long total_waves = static_cast<long>(n_wgs) * parts;
-        const int max_waves = total_waves > 32L * cus ? 8 : kMaxWaves;
-        for (int waves = 1; waves <= kMaxWaves; ++waves) {
-            if (parts % waves || parts / waves > kMaxKsplit || (eW > 0 && waves != eW) || waves < min_waves)
+    if (eCT <= 0 && nsub % kMaxWaves == 0 && N >= 16 * cus) {
+        const int SP = nsub / kMaxWaves;
+        // windows of wstride columns, r workgroups per CU
+        for (int r = (N + 64 * cus - 1) / (64 * cus); r <= 4; ++r) {
+            const int wstride = ((N + cus * r - 1) / (cus * r) + 7) / 8 * 8;
+            const int CT = (wstride + 15) / 16;
+            if (wstride < 16)
+                break;
+            if (!has_instance(CT, SP) || !shape_ok_for(MT, CT, SP) || SP > 2 * CT || CT * 16 > N)
                 continue;
-            const int ksplit = parts / waves;
-            const int U = CT * SP;
-            double cost = 0.0;
-            cost += U == want ? 0.0 : (U < want ? 2.0 * (want - U) : 1.0 * (U - want));
-            cost += 0.5 * (SP - 1);                                          // A operands per wave
-            cost += static_cast<double>(n_wgs) * CT / tiles16 - 1.0;        // columns computed twice at the edge of N
-            if (static_cast<long>(n_wgs) * ksplit < 2L * cus)
-                cost += 3.0 * (1.0 - static_cast<double>(n_wgs) * ksplit / (2.0 * cus));
-            if (waves > max_waves)
-                cost += 1.0;
-            cost -= 0.01 * waves;                                            // larger workgroups, fewer accumulations
-            if (eCT > 0 && eSP > 0 && eW > 0)
-                cost = 0.0;
-            if (cost < best_cost) {
-                best_cost = cost;
-                best = GemvPlan{CT, SP, MT, waves, n_wgs, ksplit, 0};
+            best = GemvPlan{CT, SP, MT, kMaxWaves, (N + wstride - 1) / wstride, 1, 0, wstride};
+            break;
+        }
+    }
+    if (best.CT == 0) {
+        const long units = static_cast<long>(tiles16) * nsub;
+        int want = units >= 8L * 2048 ? 8 : (units >= 4L * 2048 ? 4 : (units >= 2L * 2048 ? 2 : 1));
+        while (want > 1 && !shape_ok_for(MT, want > 4 ? 4 : want, want > 4 ? 2 : 1))
+            want /= 2;
+        double best_cost = 1e30;
+        for (int i = 0; i < kNumShapes; ++i) {
+            const int CT = kShapes[i][0], SP = kShapes[i][1];
+            if (nsub % SP || !shape_ok_for(MT, CT, SP) || CT * 16 > N)
+                continue;
+            if (eCT > 0 && eSP > 0 && (CT != eCT || SP != eSP))
+                continue;
+            const int parts = nsub / SP;             // wave-sized pieces of K
+            const int n_wgs = (tiles16 + CT - 1) / CT;
+            const long total_waves = static_cast<long>(n_wgs) * parts;
+            const int max_waves = total_waves > 32L * cus ? 8 : kMaxWaves;
+            for (int waves = 1; waves <= kMaxWaves; ++waves) {
+                if (parts % waves || parts / waves > kMaxKsplit || (eW > 0 && waves != eW) || waves < min_waves)
+                    continue;
+                const int ksplit = parts / waves;
+                const int U = CT * SP;
+                double cost = 0.0;
+                cost += U == want ? 0.0 : (U < want ? 2.0 * (want - U) : 1.0 * (U - want));
+                cost += 0.5 * (SP - 1);                                          // A operands per wave
+                cost += static_cast<double>(n_wgs) * CT / tiles16 - 1.0;        // columns computed twice at the edge of N
+                if (static_cast<long>(n_wgs) * ksplit < 2L * cus)
+                    cost += 3.0 * (1.0 - static_cast<double>(n_wgs) * ksplit / (2.0 * cus));
+                if (waves > max_waves)
+                    cost += 1.0;
+                cost -= 0.01 * waves;                                            // larger workgroups, fewer accumulations
+                if (eCT > 0 && eSP > 0 && eW > 0)
+                    cost = 0.0;
+                if (cost < best_cost) {
+                    best_cost = cost;
+                    best = GemvPlan{CT, SP, MT, waves, n_wgs, ksplit, 0, CT * 16};
+                }
             }
+        }
+        const int ews = env.wstride;
+        if (best.CT > 0 && ews > 0 && ews % 8 == 0 && ews <= best.CT * 16 && ews > (best.CT - 1) * 16) {
+            best.wstride = ews;
+            best.n_wgs = (N + ews - 1) / ews;
         }
     }
     best.lds = static_cast<size_t>(best.waves) * (2048 + (best.CT * best.MT <= 8 ? 0 : best.CT * best.MT * 256));
     return best;
+}
+
+// The plan is a function of the shape alone: kept per shape (a decode step asks for the same few shapes
+// thousands of times a second).
+GemvPlan plan_gemv(int M, int N, int K, int S, int cus, int min_waves = 1)
+{
+    struct Entry {
+        int M, N, K, S, cus, min_waves;
+        GemvPlan plan;
+    };
+    constexpr int kEntries = 64;
+    static Entry cache[kEntries];
+    static int used = 0;
+    static std::mutex lock;
+    std::lock_guard<std::mutex> guard(lock);
+    for (int i = 0; i < used; ++i) {
+        const Entry &e = cache[i];
+        if (e.M == M && e.N == N && e.K == K && e.S == S && e.cus == cus && e.min_waves == min_waves)
+            return e.plan;
+    }
+    const GemvPlan p = plan_gemv_uncached(M, N, K, S, cus, min_waves);
+    if (used < kEntries)
+        cache[used++] = Entry{M, N, K, S, cus, min_waves, p};
+    return p;
 }
 
 bool mfma_path_ok(int M, int N, int K, int S, int G)
@@ -800,6 +927,8 @@ hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, int xm, hipStrea
         return p.MT == 1 ? launch_gemv_shape<S, 1, kXAddNorm>(a, p, st) : hipErrorInvalidConfiguration;
     if (xm == kXAddNorm2)
         return p.MT == 1 ? launch_gemv_shape<S, 1, kXAddNorm2>(a, p, st) : hipErrorInvalidConfiguration;
+    if (xm == kXFloor)
+        return p.MT == 1 ? launch_gemv_shape<S, 1, kXFloor>(a, p, st) : hipErrorInvalidConfiguration;
     switch (p.MT) {
     case 1: return launch_gemv_shape<S, 1, kXPlain>(a, p, st);
 #ifndef SBVR_FAST_BUILD
@@ -1952,8 +2081,8 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
                 xm = kXAddNorm2;                                 // two chunks of x per thread
         }
         if (p.CT > 0) {
-        if (env_int("SBVR_HIP_SHOW_PLAN", 0))
-            fprintf(stderr, "sbvr_hip plan M=%d N=%d K=%d S=%d: CT=%d SP=%d MT=%d waves=%d wgs=%d ksplit=%d\n", M, N, K, S, p.CT, p.SP, p.MT, p.waves, p.n_wgs, p.ksplit);
+        if (env_switches().show_plan)
+            fprintf(stderr, "sbvr_hip plan M=%d N=%d K=%d S=%d: CT=%d SP=%d MT=%d waves=%d wgs=%d ksplit=%d wstride=%d\n", M, N, K, S, p.CT, p.SP, p.MT, p.waves, p.n_wgs, p.ksplit, p.wstride);
         GemvArgs a{};
         a.x = static_cast<const uint16_t *>(x);
         a.bvr = bvr;
@@ -1966,6 +2095,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         a.idx16 = idx_bytes == 2;
         a.ksplit = p.ksplit;
         a.xstride = pro.mode == kXSwiGLU ? 2 * K : K;
+        a.wstride = p.wstride;
         a.delta = static_cast<const uint16_t *>(pro.delta);
         a.norm_w = static_cast<const uint16_t *>(pro.norm_weight);
         a.x_out = static_cast<uint16_t *>(pro.x_out);
@@ -2071,6 +2201,15 @@ int sbvr_hip_linear_f16_add_rmsnorm(const void *x, const void *delta, const void
                        workspace_bytes, 0, stream, Prologue{kXAddNorm, delta, norm_weight, x_out, eps});
 }
 
+int sbvr_hip_linear_f16_stream_floor(const uint32_t *bvr, const void *coeff_idx, int idx_bytes,
+                                     const void *coeff_cache, void *out, int N, int K, int S, int G, int L,
+                                     void *workspace, size_t workspace_bytes, void *stream)
+{
+    // (out stands in for the activations, which this launch never reads)
+    return linear_core(out, bvr, coeff_idx, idx_bytes, coeff_cache, nullptr, out, 1, N, K, S, G, L, workspace,
+                       workspace_bytes, 0, stream, Prologue{kXFloor, nullptr, nullptr, nullptr, 0.f});
+}
+
 int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_coeff_idx,
                           int idx_bytes, const void *r_coeff_cache, const void *bias,
                           void *out, int M, int N, int K, int S, int G, int L,
@@ -2151,7 +2290,7 @@ int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_byte
         reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0 && static_cast<double>(K / 32) * N * Sr < 2147483648.0) {
         // 16-column windows (four parts of K inside a wave) when 64-column ones would leave half the CUs without a
         // workgroup: measured 13 us against 27 us at N=4096, K=14336, but 26 us against 11.5 us at N=14336, K=4096
-        const int eq = env_int("SBVR_HIP_POPC_Q", 0);
+        const int eq = env_switches().popc_q;
         const int pgrid = eq ? eq : (static_cast<long>((N + 63) / 64) * M * 2 <= current_cus() ? 4 : 1);
         const uint8_t *li = static_cast<const uint8_t *>(l_coeff_idx), *ri = static_cast<const uint8_t *>(r_coeff_idx);
         const int l16 = l_idx_bytes == 2, r16 = r_idx_bytes == 2;

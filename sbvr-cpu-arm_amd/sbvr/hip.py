@@ -49,6 +49,7 @@ def _load():
     lib.sbvr_hip_linear_f16_swiglu.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
     lib.sbvr_hip_linear_f16_add_rmsnorm.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, vp, i, vp, vp, vp,
                                                     i, i, i, i, i, vp, sz, vp]
+    lib.sbvr_hip_linear_f16_stream_floor.argtypes = [vp, vp, i, vp, vp, i, i, i, i, i, vp, sz, vp]
     lib.sbvr_hip_row_deq_mm_T.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp]
     lib.sbvr_hip_mm_T.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
     fp = ctypes.POINTER(ctypes.c_float)
@@ -208,6 +209,20 @@ def _sbvr_linear_f16_add_rmsnorm(x, delta, norm_weight, eps, x_out, bvr, coeff_i
             x.data_ptr(), delta.data_ptr(), norm_weight.data_ptr(), float(eps), x_out.data_ptr(),
             bvr.data_ptr(), coeff_idx.data_ptr(), ib, coeff_cache.data_ptr(),
             _bias_ptr(bias, N, dev), out.data_ptr(), N, K, S, G, L,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream()))
+    return out
+
+
+def _sbvr_linear_f16_stream_floor(bvr, coeff_idx, coeff_cache, bvr_len=None, out=None):
+    """Measurement aid: the one-row launch of ``_sbvr_linear_f16`` for this weight with only
+    its plane-word and index requests left in (no arithmetic, ``out`` is not written)."""
+    lib = _load()
+    dev = bvr.device
+    K = bvr.shape[0] * 32
+    N, S, G, L, ib, out, ws = _linear_operands(K, bvr, coeff_idx, coeff_cache, bvr_len, out, 1, dev)
+    with torch.cuda.device(dev):
+        _check(lib.sbvr_hip_linear_f16_stream_floor(
+            bvr.data_ptr(), coeff_idx.data_ptr(), ib, coeff_cache.data_ptr(), out.data_ptr(), N, K, S, G, L,
             ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream()))
     return out
 
