@@ -31,9 +31,13 @@ sys.path.insert(0, ROOT)
 N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH = 14336, 4096, 4, 128, 256, 1
 COPIES = 16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the gate GEMV, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# 256 MiB copy (profiles/sbvr_gemv_mfma_gate_4096x14336.txt): 29.99 MB read + 0.60 MB written.
-MEASURED_TRAFFIC_BYTES = 30.59e6
+# HBM bytes per launch of the gate GEMV as the hardware counters saw them: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy.  A profiler run's figure,
+# not measured by this script: the line names the file it comes from.
+TRAFFIC_FROM_PROFILE_BYTES = 30.59e6
+TRAFFIC_PROFILE = "profiles/sbvr_gemv_mfma_gate_4096x14336.txt"
+MIN_TIMED_LAUNCHES = 200
+_WEIGHTS = None        # the rotating weight copies on the device (built once per process)
 
 
 def algorithmic_bytes(n, k, s, g, lines, m):
@@ -42,25 +46,37 @@ def algorithmic_bytes(n, k, s, g, lines, m):
     return n * k * s // 8 + (k // g) * n * idx_bytes + 2 * lines * s + 2 * m * k + 2 * m * n
 
 
-def gpu_leg(steps, warmup):
+def gpu_leg(steps, warmup, floor=False):
+    """Times `steps` launches of the gate GEMV (or, with `floor`, of the launch that only makes its
+    memory requests), recorded into one HIP graph.  Returns the wall-clock ms per step of ONE replay
+    (the figure `value` is made from: exactly `steps` launches between two synchronisations) and the
+    HIP-event time per launch over enough further replays to cover at least MIN_TIMED_LAUNCHES
+    launches (median and minimum over the replays)."""
     import torch
     import sbvr
-    from sbvr import synth, hip
+    from sbvr import synth, hip, _sbvr_hip_ops as ops
 
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
     dev = torch.device("cuda:0")
     sbvr._sbvr_hip_init(dev)
-    weights = []
-    for c in range(COPIES):
-        bvr, idx, cache = synth.random_encoding(N_OUT, K_IN, NUM_SUMS, GROUP, LINES, seed=c)
-        weights.append((bvr.to(dev), idx.to(dev), cache.to(dev)))
+    global _WEIGHTS
+    if _WEIGHTS is None:
+        _WEIGHTS = []
+        for c in range(COPIES):
+            bvr, idx, cache = synth.random_encoding(N_OUT, K_IN, NUM_SUMS, GROUP, LINES, seed=c)
+            _WEIGHTS.append((bvr.to(dev), idx.to(dev), cache.to(dev)))
+    weights = _WEIGHTS
     x = torch.randn((BATCH, K_IN), generator=torch.Generator().manual_seed(1234)).to(torch.float16).to(dev)
     out = torch.empty((BATCH, N_OUT), dtype=torch.float16, device=dev)
 
     def step(i):
         bvr, idx, cache = weights[i % COPIES]
-        hip._sbvr_linear_f16(x, bvr, idx, cache, None, GROUP, out=out)
+        if floor:
+            hip._sbvr_linear_f16_stream_floor(bvr, idx, cache, GROUP, out=out)
+        else:
+            # the PyTorch extension over the C ABI (csrc/sbvr_ops_hip.cpp)
+            ops._sbvr_linear_f16(x, bvr, idx, cache, None, GROUP, 0, out)
 
     for i in range(warmup):
         step(i)
@@ -85,23 +101,36 @@ def gpu_leg(steps, warmup):
         graph = None
         launcher = "eager"
 
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    with torch.cuda.stream(stream):
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        e0.record(stream)
+    def run_steps():
         if graph is not None:
             graph.replay()
         else:
             for i in range(steps):
                 step(warmup + i)
-        e1.record(stream)
+
+    with torch.cuda.stream(stream):
+        # the timed region of the contract: exactly `steps` steps between two synchronisations
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_steps()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-    wall_ms = (t1 - t0) * 1e3 / steps
-    event_ms = e0.elapsed_time(e1) / steps
-    return wall_ms, event_ms, launcher, torch.cuda.get_device_name(0)
+        wall_ms = (t1 - t0) * 1e3 / steps
+        # the kernel's own time: HIP events on the launch stream around each of several replays
+        replays = max(3, -(-MIN_TIMED_LAUNCHES // steps))
+        per_launch = []
+        for _ in range(replays):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            run_steps()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            per_launch.append(e0.elapsed_time(e1) / steps)
+    per_launch.sort()
+    timing = {"median_ms": per_launch[len(per_launch) // 2], "min_ms": per_launch[0],
+              "launches_timed": replays * steps, "replays": replays}
+    return wall_ms, timing, launcher, torch.cuda.get_device_name(0)
 
 
 def decode_leg(prompt_tokens=128, new_tokens=128):
@@ -133,16 +162,55 @@ def decode_leg(prompt_tokens=128, new_tokens=128):
                  f"ffn {shape.ffn}, vocab {shape.vocab}), random init, SBVR S={NUM_SUMS} G={GROUP} on q|k|v, o, gate|up, "
                  "down; fp16 embedding and head",
         "first_tokens": [int(t) for t in tokens[:4]],
+        "breakdown_us_per_token": decode_breakdown(dec),
     }
     del dec
     torch.cuda.empty_cache()
     return out
 
 
-def _graph_time(fn, iters):
+def decode_breakdown(dec):
+    """Where a token's time goes: the three kinds of launches of a step, each recorded into a HIP graph of
+    its own (all 32 layers' worth) and replayed on the decoder's buffers after the timed generation.
+    Launches of one kind run back to back here, so the parts add up to a little less than a whole step."""
+    import torch
+    from sbvr import hip
+    s = dec.shape
+
+    def linears():
+        a, b, ctx, delta = dec.x, dec.x_alt, dec.ctx, dec.zero
+        for layer in dec.layers:
+            layer["qkv"].after_add_rmsnorm(a, delta, layer["norm1"], s.rms_eps, b)
+            delta = layer["o"](ctx)
+            gate_up = layer["gate_up"].after_add_rmsnorm(b, delta, layer["norm2"], s.rms_eps, a)
+            delta = layer["down"].after_swiglu(gate_up)
+
+    def attention():
+        for layer in dec.layers:
+            hip.dec_attention(layer["qkv"].out, dec.cos, dec.sin, dec.pos, layer["k"], layer["v"], dec.ctx,
+                              s.heads, s.kv_heads, s.head_dim, dec.rot_now)
+
+    def head():
+        hip.dec_head_argmax(dec.x, dec.zero, dec.final_norm, s.rms_eps, dec.lm_head, dec.logits, dec.tok,
+                            dec.generated, dec.pos, dec.head_ws, dec.cos, dec.sin, dec.rot_now)
+
+    parts = {"linears (4 per layer, prologues folded in)": linears, "attention (1 per layer)": attention}
+    if hip.dec_head_argmax_supported(s.hidden):
+        parts["final norm + fp16 head + argmax"] = head
+    out = {}
+    dec.reset()
+    dec.pos.fill_(dec.max_seq // 2)          # attention over half the cache, as in the middle of the timed run
+    for name, fn in parts.items():
+        out[name] = round(_graph_time(lambda i: fn(), 1, stream=dec.stream) * 1e6, 1)
+        dec.pos.fill_(dec.max_seq // 2)
+    dec.reset()
+    return out
+
+
+def _graph_time(fn, iters, stream=None):
     """Seconds per call of fn(i), i = 0..iters-1, recorded into one HIP graph and replayed (best of 3)."""
     import torch
-    stream = torch.cuda.Stream()
+    stream = stream or torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(stream):
         fn(0)
@@ -306,6 +374,24 @@ def cpu_leg(budget_s=12.0, decode=True):
     per_call = O.PORT.time_mm_T_v1(*args, warmup=10, iters=iters)
     decode_cpu = cpu_decode_estimate(threads) if decode else None
     O.PORT.finalize_pool()
+    # the same kernel on one thread (a shorter sample), and the fp16 GEMV of torch's CPU backend, which the
+    # reference's own benchmark times beside its kernel (test_sbvr.py:663-668)
+    O.PORT.init_pool(1)
+    probe1 = O.PORT.time_mm_T_v1(*args, warmup=1, iters=2)
+    one_thread = O.PORT.time_mm_T_v1(*args, warmup=2, iters=max(3, int(3.0 / max(probe1, 1e-6))))
+    O.PORT.finalize_pool()
+    import torch
+    torch.set_num_threads(threads)
+    w16 = (torch.randn((N_OUT, K_IN), generator=torch.Generator().manual_seed(3)) * 0.02).to(torch.float16)
+    x16 = torch.randn((1, K_IN), generator=torch.Generator().manual_seed(4)).to(torch.float16)
+    for _ in range(3):
+        torch.matmul(x16, w16.t())
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 2.0:
+        torch.matmul(x16, w16.t())
+        reps += 1
+    torch_gemv = (time.perf_counter() - t0) / reps
     nbytes = algorithmic_bytes(N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH)
     return {
         "value": round(nbytes / per_call / 1e9, 3),
@@ -314,6 +400,9 @@ def cpu_leg(budget_s=12.0, decode=True):
         "kind": "port",
         "us_per_gemv": round(per_call * 1e6, 1),
         "isa": O.PORT.isa(),
+        "one_thread_us": round(one_thread * 1e6, 1),
+        "torch_fp16_gemv_us": round(torch_gemv * 1e6, 1),
+        "torch_fp16_gemv_threads": threads,
         "sample": f"{iters} timed calls (10 warm-ups) of the full 4096->14336 GEMV, both operands SBVR-encoded "
                   f"(S_l=4, S_r=4, group 128), reference CPU algorithm ported to x86, N split over {threads} pinned threads",
         "decode": decode_cpu,
@@ -333,6 +422,9 @@ def main():
     ap.add_argument("--prefill", action="store_true", help="run only the prefill GEMM sizes and print them")
     ap.add_argument("--other-ops", action="store_true",
                     help="run only _sbvr_mm_T and _sbvr_row_deq_mm_T at the layer shapes and print them")
+    ap.add_argument("--stream-floor", action="store_true",
+                    help="run only the launch that makes the gate GEMV's memory requests and nothing else "
+                         "(sbvr_hip_linear_f16_stream_floor) and print its time beside the kernel's")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size kernel that "
                          "hardware byte counters are scaled by when profiling")
@@ -359,10 +451,23 @@ def main():
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
-    wall_ms, event_ms, launcher, device = gpu_leg(a.steps, a.warmup)
     nbytes = algorithmic_bytes(N_OUT, K_IN, NUM_SUMS, GROUP, LINES, BATCH)
+    _, floor_t, _, _ = gpu_leg(a.steps, a.warmup, floor=True)
+    floor = {
+        "what": "the same launch with only its plane-word and index requests (no activations, no arithmetic, no output)",
+        "us_per_launch": round(floor_t["median_ms"] * 1e3, 3),
+        "us_per_launch_min": round(floor_t["min_ms"] * 1e3, 3),
+        "frac_of_hbm_peak": round(nbytes / (floor_t["median_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+    }
+    wall_ms, timing, launcher, device = gpu_leg(a.steps, a.warmup)
+    if a.stream_floor:
+        print(json.dumps({"metric": "SBVR gate GEMV 4096->14336: kernel and its memory-request floor, us per launch",
+                          "kernel_us": round(timing["median_ms"] * 1e3, 3), "kernel_us_min": round(timing["min_ms"] * 1e3, 3),
+                          "stream_floor": floor,
+                          "kernel_over_floor": round(timing["median_ms"] / floor_t["median_ms"], 3)}))
+        return
     value = nbytes / (wall_ms * 1e-3) / 1e9
-    achieved = nbytes / (event_ms * 1e-3) / 1e9
+    achieved = nbytes / (timing["median_ms"] * 1e-3) / 1e9
     line = {
         "metric": "SBVR GEMV achieved HBM GB/s (%peak) at 4096x14336; 8B decode tokens/s",
         "value": round(value, 1),
@@ -374,7 +479,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f16 (fp8 x fp4 MFMA plane sums, f32 accumulate)",
         "data": "synthetic",
         "config": {
             "workload": "Llama-3-8B gate linear 4096->14336, batch 1, SBVR 4 bit planes, group 128, "
@@ -382,9 +487,12 @@ def main():
             "weight_copies_rotated": COPIES,
             "bytes_per_step": nbytes,
             "launcher": launcher,
+            "binding": "sbvr._sbvr_hip_ops (PyTorch extension over the C ABI)",
             "device": device,
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "clocks": "value and ms_per_step: host wall clock around one replay of `steps` launches between two "
+                  "synchronisations; roofline: HIP events on the launch stream, median over the replays",
         "roofline": {
             "bound": "hbm",
             "kernel": "sbvr_gemv_mfma_kernel",
@@ -392,10 +500,18 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "us_per_launch": round(event_ms * 1e3, 3),
-            "traffic": MEASURED_TRAFFIC_BYTES,
+            "us_per_launch": round(timing["median_ms"] * 1e3, 3),
+            "us_per_launch_min": round(timing["min_ms"] * 1e3, 3),
+            "frac_at_min": round(nbytes / (timing["min_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "launches_timed": timing["launches_timed"],
+            "traffic": TRAFFIC_FROM_PROFILE_BYTES,
+            "traffic_source": TRAFFIC_PROFILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this "
+                              "command, scaled by a 256 MiB copy; not measured in this run)",
+            "stream_floor": floor,
         },
     }
+    global _WEIGHTS
+    _WEIGHTS = None                      # (the decode leg wants the memory)
     if not a.no_decode:
         line["decode"] = decode_leg()
     if not a.no_cpu:

@@ -30,11 +30,22 @@ extern "C" {
 #define SBVR_HIP_ELAUNCH (-3)     /* HIP reported an error at launch */
 #define SBVR_HIP_EWORKSPACE (-4)  /* workspace missing or too small */
 
-/* ABI version of this header (major*100 + minor); 101 added the one-row linears with a fused prologue. */
+/* ABI version of this header (major*100 + minor); 101 added the one-row linears with a fused prologue,
+ * 102 sbvr_hip_linear_f16_stream_floor and sbvr_hip_last_kernel. */
 int sbvr_hip_version(void);
 
 /* Text of the last error raised on this thread ("" if none). */
 const char *sbvr_hip_last_error(void);
+
+/* Which kernel the last successful sbvr_hip_linear_f16* call on this thread launched (0 before the first):
+ * the routing depends on the shape and on the device (see sbvr_hip_linear_f16), and the kernels differ in
+ * how they round, so a caller or a test that cares can ask. */
+#define SBVR_HIP_KERNEL_PORTABLE 1       /* one thread per output */
+#define SBVR_HIP_KERNEL_DECODE 2         /* up to 16 rows, plane sums on the matrix cores, exact activations */
+#define SBVR_HIP_KERNEL_ROWS32 3         /* up to 32 rows, weights decoded to fp16 in registers */
+#define SBVR_HIP_KERNEL_PREFILL 4        /* weights decoded to fp16 tiles in LDS */
+#define SBVR_HIP_KERNEL_PREFILL_SPLIT 5  /* the same with K split across workgroups (workspace given) */
+int sbvr_hip_last_kernel(void);
 
 /* Checks that `device` is a gfx950 part and caches its properties.
  * Replaces sbvr_cuda_init, sbvr/kernels/sbvr_ops.cpp:122-150. */
@@ -63,19 +74,35 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  *               sbvr/kernels/sbvr_kernel.cu:555-559 does
  *   out         (M, N)      fp16
  * fp32 accumulation, one rounding to fp16.  K must be a multiple of G and G of
- * 32.  M <= 4 (M <= 16 with flags bit 1) takes the decode kernel (plane sums on
- * the matrix cores, exact fp16 activations); larger M takes the prefill kernels, which decodes weight
- * tiles to fp16 first (each decoded weight an fp16 sum of its coefficients, as
- * decode() of sbvr/core.py:927-949 rounds weights to fp16) and needs K and G to
- * be multiples of 64; other shapes fall back to the portable kernel.
+ * 32.  Which kernel runs (sbvr_hip_last_kernel() tells) depends on the shape:
+ *   decode kernel   M <= 16, N >= 16, K and G multiples of 128 with G/128 a power
+ *                   of two, S in {2,3,4,6,8}: plane sums on the matrix cores over
+ *                   the raw bit planes, the fp16 activations represented exactly;
+ *                   within 2 fp16 ulps of the exact sum.  Taken for M <= 8 always,
+ *                   and for 9..16 rows unless the 32-row kernel is preferred;
+ *   32-row kernel   5 <= M <= 32, K and G multiples of 32, same S: preferred for
+ *                   17..32 rows, for 5..16 rows of shapes the decode kernel has no
+ *                   instance for, and for 9..16 rows when N gives at least one
+ *                   32-column workgroup per CU of the device (ceil(N/32) >= CUs;
+ *                   N >= 8192 on an MI355X);
+ *   prefill kernel  M > 32 (or 17..32 with flags bit 1), K and G multiples of 64,
+ *                   same S; with a workspace and few output tiles, K is split
+ *                   across workgroups;
+ *   portable kernel everything else (one thread per output), and with flags bit 0.
+ * The 32-row and prefill kernels decode the weights to fp16 first (each decoded
+ * weight an fp16 sum of its coefficients, as decode() of sbvr/core.py:927-949
+ * rounds weights to fp16): their error is a few 1e-3 of the RMS output, within
+ * the 1e-2 relative bound for outputs that are not small against it.
  * The reference has no kernel of exactly this form (its fp16-activation
  * kernels, sbvr_kernel.cu:121-359 behind sbvr_ops.cpp:79-120, want the
  * trans=True layout); this is the operator its models/sbvr_llama.py:86-87
  * SBVRLinear.forward stands for.
- * flags: bit 0 forces the portable kernel (one thread per output); bit 1 keeps
- * the decode kernel for 5..16 rows, where the default is a 32-row MFMA kernel
- * that decodes weights to fp16 like the prefill kernel (faster there, and with
- * the prefill kernel's rounding).
+ * flags: bit 0 forces the portable kernel; bit 1 keeps the 32-row kernel out
+ * (5..16 rows then take the decode kernel, 17..32 the prefill kernel).
+ * Range: where the decode kernel splits K across workgroups, a workgroup's
+ * partial sum is clamped to +-130000 before it is added up in fixed point;
+ * partial sums beyond twice the fp16 range that would cancel to a finite total
+ * come out as a wrong finite value instead.
  */
 int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_idx,
                         int idx_bytes, const void *coeff_cache, const void *bias,

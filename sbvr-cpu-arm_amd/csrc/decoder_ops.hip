@@ -611,9 +611,15 @@ head_argmax_kernel(const uint16_t *x, const uint16_t *delta, const uint16_t *wei
         for (int w = 1; w < kHeadThreads / 64; ++w)
             key = best[w] > key ? best[w] : key;
         const unsigned long long before = __hip_atomic_fetch_max(work, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // (before & 0 ties the count to the returned value: issued only once the maximum is in place)
-        const unsigned long long count = __hip_atomic_fetch_add(work + 1, 1ull + (before & 0ull), __ATOMIC_RELAXED,
-                                                                __HIP_MEMORY_SCOPE_AGENT);
+        // The count must not be raised before this workgroup's maximum is in place: the workgroup that completes the
+        // count reads the maximum and zeroes both words.  The addend is made to depend on the value the maximum
+        // returned (the empty statement takes `before` in a register and gives `one` back as something the compiler
+        // cannot see through), so the add is issued only once that value has come back, i.e. once the maximum has
+        // been applied where all workgroups' atomics meet.  Both are returning atomics of one thread on neighbouring
+        // words; no fence is involved (an agent-scope fence writes back the XCD's whole L2).
+        unsigned long long one = 1ull;
+        asm volatile("" : "+v"(one) : "v"(before));
+        const unsigned long long count = __hip_atomic_fetch_add(work + 1, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         last = count + 1 == gridDim.x;
         if (last) {
             const unsigned long long win = __hip_atomic_load(work, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -55,6 +55,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
 thread_local char g_err[256] = "";
+thread_local int g_last_kernel = 0;       // SBVR_HIP_KERNEL_* of the last linear launched from this thread
 
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int fail(int code, const char *fmt, ...)
@@ -786,9 +787,8 @@ bool has_instance(int CT, int SP)
 //     can have in flight, so a CU with 4 workgroups where others have 3 sets the time of the whole launch
 //     (4096 -> 14336 on 256 CUs: 256 windows of 56 columns, 7.9 us against 8.6 us for 224 x 4 of 64).
 //  2. Otherwise:
-//  - about 4 units per wave when there is enough work for 2048 such waves, 8 with four times that,
-//    fewer otherwise, with as many of them as possible along N (one sub-group
-//    per wave means one set of A operands per wave);
+//  - about 4 units per wave when there is enough work for 4096 such waves, fewer otherwise, with as many
+//    of them as possible along N (one sub-group per wave means one set of A operands per wave);
 //  - at least two workgroups per CU, so K is split across workgroups (through
 //    the accumulators) when N alone does not give that many;
 //  - the largest workgroup that keeps that, but no more than 8 waves when the
@@ -801,24 +801,29 @@ GemvPlan plan_gemv_uncached(int M, int N, int K, int S, int cus, int min_waves)
     const EnvSwitches &env = env_switches();
     const int eCT = env.ct, eSP = env.sp, eW = env.waves;
     GemvPlan best{};
-    if (eCT <= 0 && nsub % kMaxWaves == 0 && N >= 16 * cus) {
-        const int SP = nsub / kMaxWaves;
+    // (with the add + norm prologue the waves of a workgroup meet at a barrier before their operands: 8-wave
+    // workgroups with four sub-groups a wave measured 14.1-14.7 us against 16.0 for 16 waves with two at
+    // 4096 -> 28672, and only that large a matrix gains from taking all of K into the workgroup)
+    const bool norm = min_waves > 1;
+    const int wg_waves = norm ? 8 : kMaxWaves;
+    if (eCT <= 0 && nsub % wg_waves == 0 && wg_waves >= min_waves && N >= (norm ? 64 : 16) * cus) {
+        const int SP = nsub / wg_waves;
         // windows of wstride columns, r workgroups per CU
         for (int r = (N + 64 * cus - 1) / (64 * cus); r <= 4; ++r) {
             const int wstride = ((N + cus * r - 1) / (cus * r) + 7) / 8 * 8;
             const int CT = (wstride + 15) / 16;
             if (wstride < 16)
                 break;
-            if (!has_instance(CT, SP) || !shape_ok_for(MT, CT, SP) || SP > 2 * CT || CT * 16 > N)
+            if (!has_instance(CT, SP) || !shape_ok_for(MT, CT, SP) || SP > (norm ? 4 : 2 * CT) || CT * 16 > N)
                 continue;
-            best = GemvPlan{CT, SP, MT, kMaxWaves, (N + wstride - 1) / wstride, 1, 0, wstride};
+            best = GemvPlan{CT, SP, MT, wg_waves, (N + wstride - 1) / wstride, 1, 0, wstride};
             break;
         }
     }
     if (best.CT == 0) {
         const long units = static_cast<long>(tiles16) * nsub;
-        int want = units >= 8L * 2048 ? 8 : (units >= 4L * 2048 ? 4 : (units >= 2L * 2048 ? 2 : 1));
-        while (want > 1 && !shape_ok_for(MT, want > 4 ? 4 : want, want > 4 ? 2 : 1))
+        int want = units >= 8L * 2048 ? 4 : (units >= 2L * 2048 ? 2 : 1);
+        while (want > 1 && !shape_ok_for(MT, want, 1))
             want /= 2;
         double best_cost = 1e30;
         for (int i = 0; i < kNumShapes; ++i) {
@@ -1971,9 +1976,11 @@ extern "C" {
 void sbvr_hip_debug_set_trace(unsigned long long *p) { g_trace = p; }
 #endif
 
-int sbvr_hip_version(void) { return 101; }      // 101: the one-row linears with a fused prologue
+int sbvr_hip_version(void) { return 102; }      // 101: the one-row linears with a fused prologue; 102: _stream_floor, last_kernel
 
 const char *sbvr_hip_last_error(void) { return g_err; }
+
+int sbvr_hip_last_kernel(void) { return g_last_kernel; }
 
 int sbvr_hip_init(int device)
 {
@@ -2066,6 +2073,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         const hipError_t e = launch_rows32(S, r, st);
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "rows32 launch: %s", hipGetErrorString(e));
+        g_last_kernel = SBVR_HIP_KERNEL_ROWS32;
         return SBVR_HIP_OK;
     }
     if ((!(flags & 1) || pro.mode != kXPlain) && aligned && mfma_path_ok(M, N, K, S, G)) {
@@ -2114,6 +2122,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         const hipError_t e = launch_gemv(S, a, p, xm, st);
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "gemv launch (CT=%d SP=%d MT=%d waves=%d ksplit=%d): %s", p.CT, p.SP, p.MT, p.waves, p.ksplit, hipGetErrorString(e));
+        g_last_kernel = SBVR_HIP_KERNEL_DECODE;
         return SBVR_HIP_OK;
         }
     }
@@ -2149,6 +2158,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         }
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "gemm launch: %s", hipGetErrorString(e));
+        g_last_kernel = g.ksplit > 1 ? SBVR_HIP_KERNEL_PREFILL_SPLIT : SBVR_HIP_KERNEL_PREFILL;
         return SBVR_HIP_OK;
     }
 
@@ -2165,6 +2175,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess)
         return fail(SBVR_HIP_ELAUNCH, "portable launch: %s", hipGetErrorString(e));
+    g_last_kernel = SBVR_HIP_KERNEL_PORTABLE;
     return SBVR_HIP_OK;
 }
 

@@ -17,6 +17,7 @@
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 #include "../../include/sbvr_hip.h"
 
@@ -65,15 +66,19 @@ void check(int rc)
 }
 
 // Zero-initialised split-K accumulators per (device, stream), grown on demand; the kernels
-// leave the part that must be zero zeroed.
+// leave the part that must be zero zeroed.  A buffer that is outgrown is kept until the process
+// ends: a HIP graph captured earlier on that stream still holds its address.
 torch::Tensor workspace(size_t nbytes, const torch::Tensor &like, hipStream_t stream)
 {
     static std::mutex mu;
     static std::map<std::tuple<int, hipStream_t>, torch::Tensor> held;
+    static std::vector<torch::Tensor> outgrown;
     std::lock_guard<std::mutex> lock(mu);
     auto key = std::make_tuple(static_cast<int>(like.get_device()), stream);
     auto it = held.find(key);
     if (it == held.end() || static_cast<size_t>(it->second.numel()) < nbytes) {
+        if (it != held.end())
+            outgrown.push_back(it->second);
         const int64_t size = static_cast<int64_t>(nbytes > (1u << 20) ? nbytes : (1u << 20));
         held[key] = torch::zeros({size}, torch::dtype(torch::kUInt8).device(like.device()));
         it = held.find(key);
@@ -115,14 +120,22 @@ void sbvr_hip_init_current()
 
 // y = x @ decode(W)^T (+ bias): x (M, K) fp16; W in the default layout, bvr (K/32, N, S) uint32,
 // coeff_idx (K/G, N), coeff_cache (L, S) fp16.  bvr_len <= 0: the group length follows from coeff_idx.
+// out: an (M, N) fp16 tensor to write into (a caller that records a HIP graph brings its own), or None.
 torch::Tensor sbvr_linear_f16(torch::Tensor x, torch::Tensor bvr, torch::Tensor coeff_idx, torch::Tensor coeff_cache,
-                              Bias bias, int64_t bvr_len, int64_t flags)
+                              Bias bias, int64_t bvr_len, int64_t flags, c10::optional<torch::Tensor> out_opt)
 {
     want(x, "x", torch::kFloat16, 2, nullptr);
     const LinearShape s = linear_shape(x.size(0), x.size(1), bvr, coeff_idx, coeff_cache, bvr_len, x);
     const DeviceGuard guard(x.device());
     hipStream_t stream = current_stream();
-    auto out = torch::empty({s.M, s.N}, torch::dtype(torch::kFloat16).device(x.device()));
+    torch::Tensor out;
+    if (out_opt.has_value() && out_opt->defined()) {
+        out = *out_opt;
+        want(out, "out", torch::kFloat16, 2, &x);
+        TORCH_CHECK(out.size(0) == s.M && out.size(1) == s.N, "out has the wrong shape");
+    } else {
+        out = torch::empty({s.M, s.N}, torch::dtype(torch::kFloat16).device(x.device()));
+    }
     const size_t need = sbvr_hip_linear_f16_workspace(s.M, s.N, s.K, s.S, s.G);
     torch::Tensor ws = need ? workspace(need, x, stream) : torch::Tensor();
     check(sbvr_hip_linear_f16(x.data_ptr(), static_cast<const uint32_t *>(bvr.data_ptr()), coeff_idx.data_ptr(), s.ib,
@@ -234,7 +247,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           py::arg("r_bvr"), py::arg("r_coeff_idx"), py::arg("r_coeff_cache"), py::arg("bias"), py::arg("use_shfl") = 0);
     m.def("_sbvr_linear_f16", &sbvr_linear_f16, "fp16 x SBVR^T over the default layout", py::arg("x"), py::arg("bvr"),
           py::arg("coeff_idx"), py::arg("coeff_cache"), py::arg("bias") = py::none(), py::arg("bvr_len") = 0,
-          py::arg("flags") = 0);
+          py::arg("flags") = 0, py::arg("out") = py::none());
+    m.def("last_kernel", &sbvr_hip_last_kernel, "which kernel the last linear call of this thread launched");
     m.def("_sbvr_linear_f16_swiglu", &sbvr_linear_f16_swiglu, "the linear of silu(gate) * up, one row", py::arg("gate_up"),
           py::arg("bvr"), py::arg("coeff_idx"), py::arg("coeff_cache"), py::arg("bias") = py::none(),
           py::arg("bvr_len") = 0);

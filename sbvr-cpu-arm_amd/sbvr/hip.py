@@ -15,6 +15,7 @@ import torch
 _LIB_NAME = "libsbvr_hip.so"
 _lib = None
 _workspaces = {}
+_outgrown = []        # workspaces that were replaced by larger ones (HIP graphs captured earlier still point at them)
 
 
 class SbvrHipError(RuntimeError):
@@ -42,6 +43,7 @@ def _load():
     vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     lib.sbvr_hip_version.restype = i
     lib.sbvr_hip_last_error.restype = ctypes.c_char_p
+    lib.sbvr_hip_last_kernel.restype = i
     lib.sbvr_hip_init.argtypes = [i]
     lib.sbvr_hip_linear_f16_workspace.restype = sz
     lib.sbvr_hip_linear_f16_workspace.argtypes = [i, i, i, i, i]
@@ -66,6 +68,14 @@ def _load():
 def _check(rc):
     if rc != 0:
         raise SbvrHipError(f"libsbvr_hip: error {rc}: {_load().sbvr_hip_last_error().decode()}")
+
+
+KERNEL_PORTABLE, KERNEL_DECODE, KERNEL_ROWS32, KERNEL_PREFILL, KERNEL_PREFILL_SPLIT = 1, 2, 3, 4, 5
+
+
+def last_kernel():
+    """Which kernel the last linear call of this thread launched (one of the KERNEL_* codes)."""
+    return _load().sbvr_hip_last_kernel()
 
 
 def _sbvr_hip_init(device=None):
@@ -115,10 +125,13 @@ def _stream():
 
 def _workspace(nbytes, device):
     """Zero-initialised scratch per (device, stream); grown on demand.  The
-    kernels leave the part that must be zero zeroed."""
+    kernels leave the part that must be zero zeroed.  A buffer that is outgrown
+    stays allocated: a HIP graph recorded earlier on the stream keeps its address."""
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is not None:
+            _outgrown.append(ws)
         ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws

@@ -4,7 +4,17 @@ intended forward is ``x @ restored_weight.T`` (:86-87); this one holds the three
 arrays of an ``sbvr`` object and calls the HIP operator."""
 import torch
 
-from . import hip, layout
+from . import layout
+
+
+def _ops():
+    """The PyTorch-ROCm extension over the library's C ABI (csrc/sbvr_ops_hip.cpp); there is no fallback."""
+    try:
+        from . import _sbvr_hip_ops
+    except ImportError as exc:
+        raise RuntimeError("sbvr._sbvr_hip_ops is not built: run `make -C sbvr-cpu-arm_amd/csrc all` "
+                           "(or __graft_entry__.build()); SBVRLinear has no other path") from exc
+    return _sbvr_hip_ops
 
 
 class SBVRLinear(torch.nn.Module):
@@ -53,6 +63,6 @@ class SBVRLinear(torch.nn.Module):
             x2 = torch.nn.functional.pad(x2, (0, self.k_padded - x2.shape[1]))
         x2 = x2.contiguous()
         # any number of rows: the operator picks the decode, 32-row or prefill kernel
-        y = hip._sbvr_linear_f16(x2, self.bvr, self.coeff_idx, self.coeff_cache, self.bias, self.bvr_len)
+        y = _ops()._sbvr_linear_f16(x2, self.bvr, self.coeff_idx, self.coeff_cache, self.bias, self.bvr_len)
         y = y[:, :self.out_features]
         return y.reshape(*lead, self.out_features)

@@ -50,6 +50,8 @@ CASES = {
     "v2_s2": ((4, 512), 2, {"cpu_kernel_v2": True}, 0.3),
     "trans_s2": ((256, 6), 2, {"trans": True}, 0.3),
     "weights_s4": ((6, 768), 4, {}, 0.02),
+    # enough rows for the MFMA kernels (they take 16 columns and more): weights ~ N(0, 0.02)
+    "weights_s4_n64": ((64, 512), 4, {}, 0.02),
 }
 
 

@@ -152,7 +152,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in sbvr_hip.h but not exported"
     lib.sbvr_hip_version.restype = ctypes.c_int
-    assert lib.sbvr_hip_version() == 101
+    assert lib.sbvr_hip_version() == 102
     lib.sbvr_hip_linear_f16_workspace.restype = ctypes.c_size_t
     assert lib.sbvr_hip_linear_f16_workspace(1, 14336, 4096, 4, 128) == 14336 * 8
     assert lib.sbvr_hip_linear_f16_workspace(1, 64, 96, 4, 32) == 0        # portable kernel: no workspace

@@ -1,29 +1,33 @@
-"""Prefill path (M > 16: weights decoded to fp16 tiles in LDS, fp16 MFMA)
-against the oracle.  The path rounds each decoded weight to fp16 (as the
-reference's decode() does, sbvr/core.py:927-949) and accumulates in fp32; the
-bar is the stated 1e-2 relative on fp16 outputs."""
+"""Prefill path (M > 32: weights decoded to fp16 tiles in LDS, fp16 MFMA) and the 32-row kernel
+(weights decoded to fp16 in registers) against the oracle.  Both round each decoded weight to fp16
+(as the reference's decode() does, sbvr/core.py:927-949) and accumulate in fp32; the bar is the
+stated 1e-2 relative on fp16 outputs, and every test names the kernel it expects to have run."""
 import numpy as np
 import pytest
 import torch
 
 pytestmark = pytest.mark.gpu
 
+DECODE, ROWS32, PREFILL, PREFILL_SPLIT = 2, 3, 4, 5
+
 
 def check(y_gpu, yd, what):
-    """1e-2 relative; outputs below half the RMS output are judged against that half.
-    Every decoded weight is an fp16 sum of up to S fp16 coefficients here (the reference's
-    decode() rounds its weights to fp16 too), so an output's error scales with the RMS
-    output, about 2e-3 of it at most, and not with its own (possibly cancelling) value."""
+    """Every decoded weight is an fp16 sum of up to S fp16 coefficients here (the reference's
+    decode() rounds its weights to fp16 too), so an output's error scales with the RMS output
+    and not with its own (possibly cancelling) value: the error must stay below 3e-3 of the RMS
+    output (2.2e-3 is the largest seen), and within 1e-2 relative for every output that is
+    not small against the RMS (those below 0.3 RMS are judged against 0.3 RMS)."""
     y = y_gpu.float().cpu().numpy().astype(np.float64)
     rms = float(np.sqrt(np.mean(yd ** 2))) + 1e-30
     err = np.abs(y - yd)
-    rel = err / np.maximum(np.abs(yd), 0.5 * rms)
+    assert err.max() <= 3e-3 * rms + 2.0 ** -11 * np.abs(yd).max(), f"{what}: error {err.max() / rms:.3e} of the RMS output"
+    rel = err / np.maximum(np.abs(yd), 0.3 * rms)
     assert rel.max() <= 1e-2, f"{what}: relative error {rel.max():.3e} > 1e-2 (abs/rms {err.max() / rms:.3e})"
 
 
-def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False):
+def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False, expect=None):
     import sbvr
-    from sbvr import synth
+    from sbvr import hip, synth
     dev = torch.device("cuda:0")
     bvr, idx, cache = synth.random_encoding(N, K, S, G, L, seed=seed)
     gen = torch.Generator().manual_seed(seed + 1)
@@ -31,31 +35,34 @@ def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False):
     b = (torch.randn((N,), generator=gen) * 0.3).to(torch.float16) if bias else None
     y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev),
                               None if b is None else b.to(dev), bvr_len=G)
+    ran = hip.last_kernel()
     torch.cuda.synchronize()
+    if expect is not None:
+        assert ran == expect, f"N={N} K={K} S={S} G={G} M={M}: kernel {ran} ran, {expect} expected"
     _, yd = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), G)
     if b is not None:
         yd = yd + b.numpy().astype(np.float64)
     check(y, yd, f"N={N} K={K} S={S} G={G} M={M} L={L}")
 
 
-@pytest.mark.parametrize("M", [17, 64, 256, 300])
+@pytest.mark.parametrize("M", [33, 64, 256, 300])
 def test_rows(oracle, M):
-    run_case(oracle, 256, 512, 4, 128, M, 256, seed=M)
+    run_case(oracle, 256, 512, 4, 128, M, 256, seed=M, expect=PREFILL)
 
 
 @pytest.mark.parametrize("S", [2, 3, 4, 6, 8])
 def test_planes(oracle, S):
-    run_case(oracle, 128, 512, S, 128, 96, 200, seed=10 + S)
+    run_case(oracle, 128, 512, S, 128, 96, 200, seed=10 + S, expect=PREFILL)
 
 
 @pytest.mark.parametrize("G", [64, 128, 256, 512])
 def test_groups(oracle, G):
-    run_case(oracle, 256, 1024, 4, G, 40, 256, seed=20 + G)
+    run_case(oracle, 256, 1024, 4, G, 40, 256, seed=20 + G, expect=PREFILL)
 
 
 @pytest.mark.parametrize("N", [16, 100, 130, 1000])
 def test_ragged_n(oracle, N):
-    run_case(oracle, N, 256, 4, 128, 33, 64, seed=30 + N)
+    run_case(oracle, N, 256, 4, 128, 33, 64, seed=30 + N, expect=PREFILL)
 
 
 @pytest.mark.parametrize("K,G", [(64, 64), (128, 64), (128, 128), (192, 64), (256, 256)])
@@ -66,37 +73,47 @@ def test_fewer_steps_than_pipeline_stages(oracle, K, G):
 
 
 def test_u16_index_and_bias(oracle):
-    run_case(oracle, 320, 768, 4, 128, 50, 3000, seed=41)
-    run_case(oracle, 320, 768, 3, 128, 50, 256, seed=42, bias=True)
+    run_case(oracle, 320, 768, 4, 128, 50, 3000, seed=41, expect=PREFILL)
+    run_case(oracle, 320, 768, 3, 128, 50, 256, seed=42, bias=True, expect=PREFILL)
 
 
 def test_two_tiles_each_way(oracle):
     run_case(oracle, 384, 1024, 4, 128, 520, 256, seed=43)
 
 
-@pytest.mark.parametrize("M", [5, 8, 16, 31, 32])
+@pytest.mark.parametrize("M", [17, 20, 31, 32])
 def test_rows32_kernel_rows(oracle, M):
-    """5..32 rows: 32-row MFMA kernel with the weights decoded in registers."""
-    run_case(oracle, 256, 512, 4, 128, M, 256, seed=70 + M)
+    """17..32 rows always take the 32-row MFMA kernel (weights decoded in registers)."""
+    run_case(oracle, 256, 512, 4, 128, M, 256, seed=70 + M, expect=ROWS32)
 
 
-@pytest.mark.parametrize("S,G", [(2, 128), (3, 128), (4, 32), (4, 64), (4, 256), (6, 128), (8, 128)])
+@pytest.mark.parametrize("M", [5, 8, 16])
+def test_rows32_kernel_few_rows_short_groups(oracle, M):
+    """5..16 rows reach it where the decode kernel has no instance (groups of 32 or 64)."""
+    run_case(oracle, 256, 512, 4, 64, M, 256, seed=170 + M, expect=ROWS32)
+
+
+@pytest.mark.parametrize("S,G", [(2, 128), (3, 128), (4, 32), (4, 64), (4, 256), (6, 128), (8, 128), (2, 32), (3, 64),
+                                 (6, 64), (8, 32)])
 def test_rows32_kernel_planes_groups(oracle, S, G):
-    run_case(oracle, 96, 768, S, G, 12, 200, seed=80 + S + G)
+    run_case(oracle, 96, 768, S, G, 19, 200, seed=80 + S + G, expect=ROWS32)
 
 
 @pytest.mark.parametrize("N,K", [(16, 256), (100, 160), (1000, 96), (130, 2048)])
 def test_rows32_kernel_ragged(oracle, N, K):
-    run_case(oracle, N, K, 4, 32, 7, 64, seed=90 + N)
+    run_case(oracle, N, K, 4, 32, 7, 64, seed=90 + N, expect=ROWS32)
 
 
 def test_rows32_kernel_u16_index_and_bias(oracle):
-    run_case(oracle, 320, 768, 4, 128, 9, 3000, seed=95)
-    run_case(oracle, 320, 768, 3, 128, 16, 256, seed=96, bias=True)
+    run_case(oracle, 320, 768, 4, 128, 21, 3000, seed=95, expect=ROWS32)
+    run_case(oracle, 320, 768, 3, 128, 32, 256, seed=96, bias=True, expect=ROWS32)
+    run_case(oracle, 320, 768, 2, 64, 9, 5000, seed=98, bias=True, expect=ROWS32)
 
 
-def test_rows32_kernel_gate_shape(oracle):
-    run_case(oracle, 14336, 4096, 4, 128, 16, 256, seed=97)
+@pytest.mark.parametrize("S", [2, 3, 4])
+def test_rows32_kernel_gate_shape(oracle, S):
+    """16 rows at 4096 -> 14336: one 32-column workgroup per CU and more, so the default is the 32-row kernel."""
+    run_case(oracle, 14336, 4096, S, 128, 16, 256, seed=97 + S, expect=ROWS32)
 
 
 def test_matches_decode_path_rows():
