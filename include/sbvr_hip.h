@@ -31,7 +31,7 @@ extern "C" {
 #define SBVR_HIP_EWORKSPACE (-4)  /* workspace missing or too small */
 
 /* ABI version of this header (major*100 + minor); 101 added the one-row linears with a fused prologue,
- * 102 sbvr_hip_linear_f16_stream_floor and sbvr_hip_last_kernel. */
+ * 102 sbvr_hip_linear_f16_noalloc and sbvr_hip_linear_f16_stream_floor. */
 int sbvr_hip_version(void);
 
 /* Text of the last error raised on this thread ("" if none). */
@@ -109,6 +109,23 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
                         void *out, int M, int N, int K, int S, int G, int L,
                         void *workspace, size_t workspace_bytes, int flags,
                         void *stream);
+
+/*
+ * sbvr_hip_linear_f16 for callers that cannot allocate device memory or bring
+ * a workspace (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  It has no counterpart in the reference.  Same
+ * arguments and results as sbvr_hip_linear_f16 without the workspace pair: the
+ * decode kernel's split-K accumulators live in a 4 MiB array inside the
+ * library (one copy per GPU, held until the process ends), so up to 16 rows
+ * need M * N <= 524288 (SBVR_HIP_EWORKSPACE beyond that); with more rows the
+ * prefill kernel runs without its optional workspace, i.e. not split along K.
+ * The call allocates and frees nothing.  Calls that overlap in time on one GPU
+ * share the array and race: serialise them (one stream, or events).
+ */
+int sbvr_hip_linear_f16_noalloc(const void *x, const uint32_t *bvr, const void *coeff_idx,
+                                int idx_bytes, const void *coeff_cache, const void *bias,
+                                void *out, int M, int N, int K, int S, int G, int L,
+                                int flags, void *stream);
 
 /*
  * The same operator for one row (M = 1) with the elementwise step that feeds

@@ -1968,6 +1968,40 @@ bool launch_mm_T_popc_sr(int Sr, int Q, hipStream_t st, const uint32_t *l_bvr, c
 
 } // namespace
 
+// Scratch memory of sbvr_hip_linear_f16_noalloc: the split-K accumulators of the decode kernel, for callers
+// that cannot bring a workspace.  One copy per GPU the library runs on, held until the process ends; zero when
+// the module is loaded, and every launch leaves it zero (the adder that completes an accumulator resets it).
+// In host code the array's name is only a handle: its device address is asked for once per device
+// (scratch_on_current_device) and that pointer is what launches get.
+constexpr size_t kScratchBytes = 4u << 20;       // 524288 accumulators: M * N of the largest decode launch it takes
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+
+void *g_scratch_ptr[16] = {};
+
+// Device address of `scratch` on the current device (looked up on first use, with that device current).
+int scratch_on_current_device(void **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return fail(SBVR_HIP_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= 16)
+        return fail(SBVR_HIP_EUNSUPPORTED, "device %d: this library keeps scratch memory for devices 0..15", dev);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(SBVR_HIP_ELAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return SBVR_HIP_OK;
+}
+
+} // namespace
+
 // ------------------------------------------------------------------- C ABI
 
 extern "C" {
@@ -1976,7 +2010,7 @@ extern "C" {
 void sbvr_hip_debug_set_trace(unsigned long long *p) { g_trace = p; }
 #endif
 
-int sbvr_hip_version(void) { return 102; }      // 101: the one-row linears with a fused prologue; 102: _stream_floor, last_kernel
+int sbvr_hip_version(void) { return 102; }      // 101: the one-row linears with a fused prologue; 102: _noalloc, _stream_floor
 
 const char *sbvr_hip_last_error(void) { return g_err; }
 
@@ -1999,7 +2033,17 @@ int sbvr_hip_init(int device)
                     device, prop.gcnArchName);
     g_dev[device].cus = prop.multiProcessorCount;
     g_dev[device].ready = true;
-    return SBVR_HIP_OK;
+    // the scratch array's address on this device (each GPU holds its own copy at its own address)
+    int before = 0;
+    if (hipGetDevice(&before) != hipSuccess)
+        before = device;
+    if (before != device && hipSetDevice(device) != hipSuccess)
+        return fail(SBVR_HIP_ELAUNCH, "hipSetDevice(%d) failed", device);
+    void *ptr = nullptr;
+    const int rc = scratch_on_current_device(&ptr);
+    if (before != device)
+        (void)hipSetDevice(before);
+    return rc;
 }
 
 size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G)
@@ -2191,6 +2235,29 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
 {
     return linear_core(x, bvr, coeff_idx, idx_bytes, coeff_cache, bias, out, M, N, K, S, G, L, workspace,
                        workspace_bytes, flags, stream, Prologue{kXPlain, nullptr, nullptr, nullptr, 0.f});
+}
+
+int sbvr_hip_linear_f16_noalloc(const void *x, const uint32_t *bvr, const void *coeff_idx,
+                                int idx_bytes, const void *coeff_cache, const void *bias,
+                                void *out, int M, int N, int K, int S, int G, int L,
+                                int flags, void *stream)
+{
+    // The decode kernel's accumulators come from the library's own scratch array; the prefill kernel runs
+    // without its optional workspace (not split along K).  Nothing is allocated or freed on the way.
+    void *ws = nullptr;
+    size_t ws_bytes = 0;
+    if (M >= 1 && N >= 1 && mfma_path_ok(M, N, K, S, G) && !(flags & 1)) {
+        const size_t need = static_cast<size_t>(M) * N * sizeof(unsigned long long);
+        if (need > kScratchBytes)
+            return fail(SBVR_HIP_EWORKSPACE, "sbvr_hip_linear_f16_noalloc takes M * N <= %zu for up to 16 rows (M=%d N=%d); "
+                        "use sbvr_hip_linear_f16 with a workspace", kScratchBytes / sizeof(unsigned long long), M, N);
+        const int rc = scratch_on_current_device(&ws);
+        if (rc != SBVR_HIP_OK)
+            return rc;
+        ws_bytes = kScratchBytes;
+    }
+    return linear_core(x, bvr, coeff_idx, idx_bytes, coeff_cache, bias, out, M, N, K, S, G, L, ws, ws_bytes, flags,
+                       stream, Prologue{kXPlain, nullptr, nullptr, nullptr, 0.f});
 }
 
 int sbvr_hip_linear_f16_swiglu(const void *gate_up, const uint32_t *bvr, const void *coeff_idx,

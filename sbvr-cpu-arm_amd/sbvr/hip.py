@@ -51,6 +51,7 @@ def _load():
     lib.sbvr_hip_linear_f16_swiglu.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
     lib.sbvr_hip_linear_f16_add_rmsnorm.argtypes = [vp, vp, vp, ctypes.c_float, vp, vp, vp, i, vp, vp, vp,
                                                     i, i, i, i, i, vp, sz, vp]
+    lib.sbvr_hip_linear_f16_noalloc.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, vp]
     lib.sbvr_hip_linear_f16_stream_floor.argtypes = [vp, vp, i, vp, vp, i, i, i, i, i, vp, sz, vp]
     lib.sbvr_hip_row_deq_mm_T.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp]
     lib.sbvr_hip_mm_T.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
