@@ -245,16 +245,27 @@ __device__ __forceinline__ Planes<S> load_planes(const uint32_t *p)
     return r;
 }
 
-// Waves per SIMD the register allocator is asked to leave room for: the queued
-// plane words, line indices and coefficients of all units, the activations, the
-// plane sums, the A operands and working registers.
+// Waves per SIMD the register allocator is asked to leave room for: the A operands and the activations
+// they are made from, the results, the MFMA outputs and plane sums of a unit, the plane words in flight
+// and working registers.
 constexpr int gemv_waves(int S, int MT, int CT, int SP)
 {
-    const int U = CT * SP;
-    const int regs = U * (S + 1 + (S + 1) / 2) + U * MT * S + 8 * SP * MT + 4 * SP * MT + 4 * MT * S + CT * MT + 32;
+    const int regs = 12 * SP * MT + CT * MT + 5 * MT * S + 3 * S + 4 * S + 48;
     const int w = 512 / regs;
     return w < 1 ? 1 : (w > 8 ? 8 : w);
 }
+
+// Waves of a workgroup at most: 16, or 8 for the instances that want more than 128 registers a lane
+// (four row tiles, or 8 and more column tiles).
+constexpr int gemv_max_waves(int MT, int CT)
+{
+    return MT == 4 || CT > 4 ? 8 : kMaxWaves;
+}
+
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef short v2s __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ v2h as_v2h(uint32_t u) { return __builtin_bit_cast(v2h, u); }
+__device__ __forceinline__ int as_int(v2s b) { return __builtin_bit_cast(int, b); }
 
 // max over the 64 lanes of a non-negative integer; the result is wave-uniform
 __device__ __forceinline__ uint32_t wave_umax(uint32_t v)
@@ -352,7 +363,7 @@ __device__ __forceinline__ long long to_fixed(float y)
 //   5. coefficients applied; partial results to LDS, barrier, summed in a fixed
 //      order by the first waves, written out (or added to the split-K words).
 template <int S, int MT, int CT, int SP, int XM>
-__global__ void __launch_bounds__(64 * kMaxWaves)
+__global__ void __launch_bounds__(64 * gemv_max_waves(MT, CT))
 __attribute__((amdgpu_waves_per_eu(gemv_waves(S, MT, CT, SP), 8)))
 sbvr_gemv_mfma_kernel(const GemvArgs a)
 {
@@ -423,20 +434,22 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
         for (int sgi = 0; sgi < SP; ++sgi)
             xw[sgi] = reinterpret_cast<const uint32_t *>(a.norm_w + static_cast<size_t>(sg0 + sgi) * kSub)[lane];
     }
-    // line indices: one load per sub-group, lane l takes the index of column n_base + l of the
-    // window (16*CT <= 64 columns); they are handed to the (tile, column) lanes later, in LDS
-    // permutes: every vector-memory instruction saved is tens of nanoseconds of issue time
-    int lraw[SP];
-    {
-        const uint32_t lane_i = static_cast<uint32_t>(n_base + min(lane, 16 * CT - 1));
+    // line indices: one load per sub-group and 64 columns of the window, lane l takes the index of column
+    // n_base + 64*iw + l; they are handed to the (tile, column) lanes later, in LDS permutes: every
+    // vector-memory instruction saved is tens of nanoseconds of issue time
+    constexpr int IW = (16 * CT + 63) / 64;
+    int lraw[SP][IW];
+#pragma unroll
+    for (int iw = 0; iw < IW; ++iw) {
+        const uint32_t lane_i = static_cast<uint32_t>(n_base + min(64 * iw + lane, 16 * CT - 1));
         if (a.idx16) {
 #pragma unroll
             for (int sgi = 0; sgi < SP; ++sgi)
-                lraw[sgi] = static_cast<const uint16_t *>(a.idx)[static_cast<size_t>((sg0 + sgi) >> a.gshift) * N + lane_i];
+                lraw[sgi][iw] = static_cast<const uint16_t *>(a.idx)[static_cast<size_t>((sg0 + sgi) >> a.gshift) * N + lane_i];
         } else {
 #pragma unroll
             for (int sgi = 0; sgi < SP; ++sgi)
-                lraw[sgi] = static_cast<const uint8_t *>(a.idx)[static_cast<size_t>((sg0 + sgi) >> a.gshift) * N + lane_i];
+                lraw[sgi][iw] = static_cast<const uint8_t *>(a.idx)[static_cast<size_t>((sg0 + sgi) >> a.gshift) * N + lane_i];
         }
     }
     Planes<S> q[U];
@@ -456,7 +469,9 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
         uint32_t seen = 0;
 #pragma unroll
         for (int sgi = 0; sgi < SP; ++sgi)
-            seen ^= static_cast<uint32_t>(lraw[sgi]);
+#pragma unroll
+            for (int iw = 0; iw < IW; ++iw)
+                seen ^= static_cast<uint32_t>(lraw[sgi][iw]);
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -471,16 +486,21 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     // requests at a time and hands the free places to its oldest waves first: a wave that asked for all of its
     // units at once would sit in the issue of its loads for microseconds (the youngest waves until the launch
     // is nearly over) and make its operands only after that.
-    constexpr int kPre = U < kUnitsAhead ? U : kUnitsAhead;
+    // (workgroups of at most 8 waves keep twice as many, for the same number of requests per CU)
+#ifndef SBVR_AHEAD_WIDE
+#define SBVR_AHEAD_WIDE 6
+#endif
+    constexpr int kAhead = MT > 1 && CT > 4 ? SBVR_AHEAD_WIDE : (gemv_max_waves(MT, CT) == 8 ? 2 * kUnitsAhead : kUnitsAhead);
+    constexpr int kPre = U < kAhead ? U : kAhead;
     request_units(0, kPre);
     __builtin_amdgcn_sched_barrier(0);       // these requests are out before anything waits
     SBVR_STAMP(1);
 
-    // -- 2. A operands.  Lane l turns elements 2l and 2l+1 of a batch row into
-    //       3 fp8 terms each and drops the bytes where the MFMA wants them; the
-    //       lane then reads its 32 bytes back.  Row tiles go from the last one,
-    //       the only one that may have fewer than 4 rows, to the first, so a row
-    //       of the buffer that is not rewritten holds zeros.
+    // -- 2. A operands.  A lane turns two elements of a batch row into 3 fp8
+    //       terms each and drops the bytes where the MFMA wants them; the lane
+    //       then reads its 32 bytes back.  Row tiles go from the last one, the
+    //       only one that may have fewer than 4 rows, to the first, so a row of
+    //       the buffer that is not rewritten holds zeros.
     float inv = 0.f;             // with the norm: rsqrt(mean((x + delta)^2) + eps)
     if constexpr (kNorm) {
         float ss = 0.f;
@@ -531,8 +551,12 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     v8i A[SP][MT];
     float scale[SP][MT];         // of this lane's batch row (blk)
     const int m_rows = XM != kXPlain ? 1 : a.M;
-    const int off0 = a_image_byte_offset(2 * lane, 0), off1 = a_image_byte_offset(2 * lane + 1, 0);
-    const float fac0 = (lane & 1) ? 1.f : 4.f, fac1 = (lane & 1) ? 1.f : 2.f;
+    // Lane l = 4g + t of a row's 64 takes elements 8g + t and 8g + t + 4 of the sub-group: the same bit t of two
+    // neighbouring nibbles of a plane word, which are neighbouring bytes of the A image (one 16-bit store per
+    // term) and share the weight of their B digits (0.5, 1, 2, 2 for t = 0..3, made up for here: 4, 2, 1, 1).
+    const int off = a_image_byte_offset(8 * (lane >> 2) + (lane & 3), 0);
+    const uint32_t half_sel = (lane & 1) ? 0x07060302u : 0x05040100u;      // (odd t: the high halves of the dwords)
+    const int fac_log2 = (lane & 3) == 0 ? 2 : ((lane & 3) == 1 ? 1 : 0);
     // the operands of sub-groups [s0, s1) of this wave
     auto make_operands = [&](int s0, int s1) __attribute__((always_inline)) {
 #pragma unroll
@@ -557,25 +581,27 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
                         const uint32_t amax = wave_umax(max(v & 0x7fffu, (v >> 16) & 0x7fffu));
                         const int eh = min(max(static_cast<int>(amax >> 10), 1), 30);
                         const int e = 20 - eh;
-                        const float up = __uint_as_float(static_cast<uint32_t>(e + 127) << 23);
                         if (blk == r)            // products come out as 2 * x * 2^e
                             scale[sgi][mt] = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
-                        float z0 = h2f(static_cast<uint16_t>(v & 0xffffu)) * (up * fac0);
-                        float z1 = h2f(static_cast<uint16_t>(v >> 16)) * (up * fac1);
-                        // h1 + h2 + h3/256 == z exactly: each fp8 takes the next 4 significant
-                        // bits, the last one of the residual scaled up out of the subnormals
-#pragma unroll
-                        for (int term = 0; term < 3; ++term) {
-                            if (term == 2) {
-                                z0 *= kLastTermScale;
-                                z1 *= kLastTermScale;
-                            }
-                            const int b = __builtin_amdgcn_cvt_pk_fp8_f32(z0, z1, 0, false);
-                            z0 -= __builtin_amdgcn_cvt_f32_fp8(b, 0);
-                            z1 -= __builtin_amdgcn_cvt_f32_fp8(b, 1);
-                            mine[off0 + (r * 4 + term) * 32] = static_cast<unsigned char>(b & 0xff);
-                            mine[off1 + (r * 4 + term) * 32] = static_cast<unsigned char>((b >> 8) & 0xff);
-                        }
+                        // the lane's two elements, from the dwords (2l, 2l + 1) the lanes of its quad loaded
+                        const int va = __builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x50, 0xF, 0xF, true);   // quad_perm 0,0,1,1
+                        const int vb = __builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xFA, 0xF, 0xF, true);   // quad_perm 2,2,3,3
+                        v2h z = as_v2h(__builtin_amdgcn_perm(static_cast<uint32_t>(vb), static_cast<uint32_t>(va), half_sel));
+                        // h1 + h2 + h3/256 == z * 2^e * weight exactly: each fp8 takes the next 4 significant bits
+                        // (the conversions divide by their scale operand), the last one of the residual scaled up
+                        // out of the subnormals; the residuals are exact in fp16
+                        const float sc = __uint_as_float(static_cast<uint32_t>(127 - e - fac_log2) << 23);
+                        const float sc_last = __uint_as_float(static_cast<uint32_t>(127 - 8 - e - fac_log2) << 23);
+                        static_assert(kLastTermScale == 256.f, "the last term's scale is 2^8 here");
+                        v2s b = {0, 0};
+                        b = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(b, z, sc, false);
+                        z -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(as_int(b), sc, false);
+                        b = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(b, z, sc, true);
+                        z -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(as_int(b), sc, true);
+                        const v2s b3 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(v2s{0, 0}, z, sc_last, false);
+                        *reinterpret_cast<short *>(mine + off + (r * 4 + 0) * 32) = b[0];
+                        *reinterpret_cast<short *>(mine + off + (r * 4 + 1) * 32) = b[1];
+                        *reinterpret_cast<short *>(mine + off + (r * 4 + 2) * 32) = b3[0];
                     }
                 }
                 A[sgi][mt] = *reinterpret_cast<const v8i *>(mine + lane * 32);
@@ -589,35 +615,72 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     // -- 3. coefficient lines (S fp16 each): lane l gathers the line of column n_base + l for each
     //       sub-group, then the (tile, column) lanes pick theirs up with LDS permutes
     constexpr int CW = (S + 1) / 2;          // dwords per line
-    uint32_t cl[SP][CW];
+    uint32_t cl[SP][IW][CW];
 #pragma unroll
-    for (int sgi = 0; sgi < SP; ++sgi) {
-        const uint32_t line = static_cast<uint32_t>(min(lraw[sgi], a.L - 1));
-        const uint16_t *p = a.cache + line * S;
-        if constexpr (S == 4) {
-            const uint2 t = *reinterpret_cast<const uint2 *>(p);
-            cl[sgi][0] = t.x; cl[sgi][1] = t.y;
-        } else if constexpr (S == 8) {
-            const uint4 t = *reinterpret_cast<const uint4 *>(p);
-            cl[sgi][0] = t.x; cl[sgi][1] = t.y; cl[sgi][2] = t.z; cl[sgi][3] = t.w;
-        } else if constexpr (S % 2 == 0) {
+    for (int sgi = 0; sgi < SP; ++sgi)
 #pragma unroll
-            for (int j = 0; j < CW; ++j)
-                cl[sgi][j] = reinterpret_cast<const uint32_t *>(p)[j];
-        } else {
+        for (int iw = 0; iw < IW; ++iw) {
+            const uint32_t line = static_cast<uint32_t>(min(lraw[sgi][iw], a.L - 1));
+            const uint16_t *p = a.cache + line * S;
+            if constexpr (S == 4) {
+                const uint2 t = *reinterpret_cast<const uint2 *>(p);
+                cl[sgi][iw][0] = t.x; cl[sgi][iw][1] = t.y;
+            } else if constexpr (S == 8) {
+                const uint4 t = *reinterpret_cast<const uint4 *>(p);
+                cl[sgi][iw][0] = t.x; cl[sgi][iw][1] = t.y; cl[sgi][iw][2] = t.z; cl[sgi][iw][3] = t.w;
+            } else if constexpr (S % 2 == 0) {
 #pragma unroll
-            for (int j = 0; j < CW; ++j)
-                cl[sgi][j] = static_cast<uint32_t>(p[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(p[2 * j + 1]) << 16 : 0u);
+                for (int j = 0; j < CW; ++j)
+                    cl[sgi][iw][j] = reinterpret_cast<const uint32_t *>(p)[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < CW; ++j)
+                    cl[sgi][iw][j] = static_cast<uint32_t>(p[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(p[2 * j + 1]) << 16 : 0u);
+            }
         }
-    }
     SBVR_STAMP(3);
 
-    // -- 4. the units: plane sums of every (unit, row tile, plane)
-    float ps[U][MT][S];
+    // -- 4. the units: plane sums of every (unit, row tile, plane), and one unit behind them
+    // -- 5. coefficients and scales: the lane holds column n_base + 16*ct + col of batch row 4*mt + blk.
+    //       The coefficients of unit u - 1 are applied behind the MFMAs of unit u: arithmetic that does not
+    //       depend on them, for the time they take; and only one unit's plane sums are alive at a time.
+    float y[CT][MT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            y[ct][mt] = 0.f;
+    float ps[MT][S];                 // plane sums of the unit before the one in the matrix cores
+    uint32_t cqu[CW];                // and that unit's coefficient line, on its way through the LDS permute
+    // (the lane that gathered the line of column 16*ct + col of the window hands it over)
+    auto fetch_coefficients = [&](int u) __attribute__((always_inline)) {
+        const int sgi = u / CT, ct = u % CT;
+#pragma unroll
+        for (int j = 0; j < CW; ++j)
+            cqu[j] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(((ct * 16 + col) & 63) * 4,
+                                                                          static_cast<int>(cl[sgi][(ct * 16) / 64][j])));
+    };
+    auto apply_coefficients = [&](int u) __attribute__((always_inline)) {
+        const int sgi = u / CT, ct = u % CT;
+        float c[S];
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+            c[j] = h2f(static_cast<uint16_t>(j & 1 ? cqu[j / 2] >> 16 : cqu[j / 2] & 0xffffu));
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < S; ++j)
+                acc = fmaf(c[j], ps[mt][j], acc);
+            y[ct][mt] = fmaf(acc, scale[sgi][mt], y[ct][mt]);
+        }
+    };
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int sgi = u / CT;
         request_units(u + kPre, u + kPre + 1);      // keeps kPre units of this wave in flight
+        if (u > 0)
+            fetch_coefficients(u - 1);              // (on its way while this unit's operands are made)
         __builtin_amdgcn_sched_barrier(0);
         v4f D[MT][S];
 #pragma unroll
@@ -635,46 +698,21 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
                 D[mt][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[sgi][mt], B, z, 0, 4, 0, 0, 0, 0);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if (u > 0)
+            apply_coefficients(u - 1);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int j = 0; j < S; ++j) {
-                ps[u][mt][j] = fmaf(D[mt][j][2], 1.f / kLastTermScale, D[mt][j][0] + D[mt][j][1]);
-                asm volatile("" : "+v"(ps[u][mt][j]));       // keeps the units in program order
+                ps[mt][j] = fmaf(D[mt][j][2], 1.f / kLastTermScale, D[mt][j][0] + D[mt][j][1]);
+                asm volatile("" : "+v"(ps[mt][j]));          // keeps the units in program order
             }
         __builtin_amdgcn_sched_barrier(0);
     }
+    fetch_coefficients(U - 1);
+    apply_coefficients(U - 1);
     SBVR_STAMP(4);
-
-    // -- 5. coefficients and scales; the lane holds column n_base + 16*ct + col
-    //       of batch row 4*mt + blk
-    float y[CT][MT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            y[ct][mt] = 0.f;
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const int sgi = u / CT, ct = u % CT;
-        // (the permutes sit here, behind the units: the gathered lines are the youngest loads)
-        uint32_t cqu[CW];
-#pragma unroll
-        for (int j = 0; j < CW; ++j)
-            cqu[j] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute((ct * 16 + col) * 4, static_cast<int>(cl[sgi][j])));
-        float c[S];
-#pragma unroll
-        for (int j = 0; j < S; ++j)
-            c[j] = h2f(static_cast<uint16_t>(j & 1 ? cqu[j / 2] >> 16 : cqu[j / 2] & 0xffffu));
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            float acc = 0.f;
-#pragma unroll
-            for (int j = 0; j < S; ++j)
-                acc = fmaf(c[j], ps[u][mt][j], acc);
-            y[ct][mt] = fmaf(acc, scale[sgi][mt], y[ct][mt]);
-        }
-    }
     //       partial results meet in LDS: wave w's buffer holds [ct][mt][lane] floats
     // (up to 8 blocks per wave they fit the wave's own 2 KiB buffer; more go behind the buffers of all waves,
     // because another wave may still be building operands in its buffer)
@@ -759,17 +797,22 @@ const EnvSwitches &env_switches()
     return e;
 }
 
-// (CT, SP) pairs that have a kernel instance; see the dispatch below.
-constexpr int kShapes[][2] = {{1, 1}, {1, 2}, {1, 4}, {1, 7}, {2, 1}, {2, 2}, {2, 4}, {2, 7}, {4, 1}, {4, 2}, {4, 4}};
+// (CT, SP) pairs that have a kernel instance; see the dispatch below.  The wide ones (8 column tiles and
+// more) exist for 5..16 batch rows only: there every batch row of a sub-group costs a wave that uses it
+// some 55 VALU instructions of operand preparation, so a wave should use its operands for many columns.
+constexpr int kShapes[][2] = {{1, 1}, {1, 2}, {1, 4}, {1, 7}, {2, 1}, {2, 2}, {2, 4}, {2, 7}, {4, 1}, {4, 2}, {4, 4},
+                              {8, 1}, {8, 2}, {14, 1}, {16, 1}};
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
 
-bool shape_ok_for(int MT, int CT, int SP)
+constexpr bool shape_ok_for(int MT, int CT, int SP)
 {
-    // larger batches keep to the smaller unit counts (register budget)
+    if (CT > 4)             // registers: A operands 8 * SP * MT, results CT * MT
+        return MT > 1 && SP * MT <= 8 && CT * MT <= 64;
     // (the partial results of a wave, CT*MT*64 floats, fit its 2 KiB buffer up to CT*MT = 8 and get room
-    // of their own beyond: four tiles at 9..16 rows are 14 % faster than two, the operands being made once
-    // per wave whatever its tiles)
-    return CT * MT <= 16 && (MT == 1 || CT * SP * MT <= 16);
+    // of their own beyond)
+    // (two row tiles with a 16-wave launch bound, 128 registers: at most 4 sub-groups of operands, and 4 only
+    // with one column tile)
+    return CT * MT <= 16 && (MT == 1 || CT * SP * MT <= 16) && (MT != 2 || (SP <= 4 && CT * SP <= 8 && !(SP == 4 && CT > 1)));
 }
 
 bool has_instance(int CT, int SP)
@@ -801,12 +844,42 @@ GemvPlan plan_gemv_uncached(int M, int N, int K, int S, int cus, int min_waves)
     const EnvSwitches &env = env_switches();
     const int eCT = env.ct, eSP = env.sp, eW = env.waves;
     GemvPlan best{};
+    if (MT > 1 && eCT <= 0) {
+        // 5..16 batch rows: a wave's time is its operand preparation (55 VALU instructions per batch row and
+        // sub-group) plus its units (20 + 13 per row tile, and four MFMAs of 32 clocks per row tile, about half
+        // of which hide behind the VALU work): the shape with the smallest estimate of the busiest SIMD's time,
+        // workgroups of up to 8 waves for the wide shapes (they hold up to 256 registers a lane).
+        double best_t = 1e30;
+        for (int i = 0; i < kNumShapes; ++i) {
+            const int CT = kShapes[i][0], SP = kShapes[i][1];
+            if (nsub % SP || !shape_ok_for(MT, CT, SP) || CT * 16 > N)
+                continue;
+            const int parts = nsub / SP;
+            const int windows = (tiles16 + CT - 1) / CT;
+            const int wave_cap = gemv_max_waves(MT, CT);
+            for (int waves = 1; waves <= wave_cap; ++waves) {
+                if (parts % waves || parts / waves > kMaxKsplit)
+                    continue;
+                const int ksplit = parts / waves;
+                const long wgs = static_cast<long>(windows) * ksplit;
+                const long rounds = (wgs + cus - 1) / cus;                       // workgroups the busiest CU runs
+                const double per_wave = 55.0 * SP * M + static_cast<double>(CT) * SP * (20.0 + 13.0 * MT + 16.0 * MT);
+                double t = static_cast<double>(rounds) * ((waves + 3) / 4) * per_wave;
+                t += 0.02 * static_cast<double>(M) * N * ksplit / cus;          // the accumulators' atomics
+                t *= static_cast<double>(windows) * CT / tiles16;               // columns computed for nothing at the edge
+                if (t < best_t) {
+                    best_t = t;
+                    best = GemvPlan{CT, SP, MT, waves, windows, ksplit, 0, CT * 16};
+                }
+            }
+        }
+    }
     // (with the add + norm prologue the waves of a workgroup meet at a barrier before their operands: 8-wave
     // workgroups with four sub-groups a wave measured 14.1-14.7 us against 16.0 for 16 waves with two at
     // 4096 -> 28672, and only that large a matrix gains from taking all of K into the workgroup)
     const bool norm = min_waves > 1;
     const int wg_waves = norm ? 8 : kMaxWaves;
-    if (eCT <= 0 && nsub % wg_waves == 0 && wg_waves >= min_waves && N >= (norm ? 64 : 16) * cus) {
+    if (best.CT == 0 && eCT <= 0 && nsub % wg_waves == 0 && wg_waves >= min_waves && N >= (norm ? 64 : 16) * cus) {
         const int SP = nsub / wg_waves;
         // windows of wstride columns, r workgroups per CU
         for (int r = (N + 64 * cus - 1) / (64 * cus); r <= 4; ++r) {
@@ -836,7 +909,7 @@ GemvPlan plan_gemv_uncached(int M, int N, int K, int S, int cus, int min_waves)
             const int n_wgs = (tiles16 + CT - 1) / CT;
             const long total_waves = static_cast<long>(n_wgs) * parts;
             const int max_waves = total_waves > 32L * cus ? 8 : kMaxWaves;
-            for (int waves = 1; waves <= kMaxWaves; ++waves) {
+            for (int waves = 1; waves <= gemv_max_waves(MT, CT); ++waves) {
                 if (parts % waves || parts / waves > kMaxKsplit || (eW > 0 && waves != eW) || waves < min_waves)
                     continue;
                 const int ksplit = parts / waves;
@@ -904,6 +977,19 @@ template <int S, int MT, int CT, int SP, int XM>
 hipError_t launch_gemv_inst(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
     const dim3 grid(static_cast<unsigned>(p.n_wgs), static_cast<unsigned>(p.ksplit)), block(64 * p.waves);
+    if (p.lds > 65536) {        // (the wide shapes' partial results) above what a kernel gets without asking
+        static bool raised_on[16] = {};
+        int dev_now = 0;
+        if (hipGetDevice(&dev_now) != hipSuccess || dev_now < 0 || dev_now >= 16)
+            dev_now = 0;
+        if (!raised_on[dev_now]) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sbvr_gemv_mfma_kernel<S, MT, CT, SP, XM>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess)
+                return e;
+            raised_on[dev_now] = true;
+        }
+    }
     hipLaunchKernelGGL((sbvr_gemv_mfma_kernel<S, MT, CT, SP, XM>), grid, block, p.lds, st, a);
     return hipGetLastError();
 }
@@ -912,12 +998,13 @@ template <int S, int MT, int XM>
 hipError_t launch_gemv_shape(const GemvArgs &a, const GemvPlan &p, hipStream_t st)
 {
 #define SBVR_SHAPE(ct, sp)                                  \
-    if constexpr (ct * MT <= 16 && (ct * sp * MT <= 16 || MT == 1)) \
+    if constexpr (shape_ok_for(MT, ct, sp))                 \
         if (p.CT == ct && p.SP == sp)                       \
             return launch_gemv_inst<S, MT, ct, sp, XM>(a, p, st)
     SBVR_SHAPE(1, 1); SBVR_SHAPE(1, 2); SBVR_SHAPE(1, 4); SBVR_SHAPE(1, 7);
     SBVR_SHAPE(2, 1); SBVR_SHAPE(2, 2); SBVR_SHAPE(2, 4); SBVR_SHAPE(2, 7);
     SBVR_SHAPE(4, 1); SBVR_SHAPE(4, 2); SBVR_SHAPE(4, 4);
+    SBVR_SHAPE(8, 1); SBVR_SHAPE(8, 2); SBVR_SHAPE(14, 1); SBVR_SHAPE(16, 1);
 #undef SBVR_SHAPE
     return hipErrorInvalidConfiguration;
 }
@@ -936,12 +1023,8 @@ hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, int xm, hipStrea
         return p.MT == 1 ? launch_gemv_shape<S, 1, kXFloor>(a, p, st) : hipErrorInvalidConfiguration;
     switch (p.MT) {
     case 1: return launch_gemv_shape<S, 1, kXPlain>(a, p, st);
-#ifndef SBVR_FAST_BUILD
     case 2: return launch_gemv_shape<S, 2, kXPlain>(a, p, st);
     default: return launch_gemv_shape<S, 4, kXPlain>(a, p, st);
-#else
-    default: return hipErrorInvalidConfiguration;
-#endif
     }
 }
 
