@@ -78,13 +78,12 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  *   decode kernel   M <= 16, N >= 16, K and G multiples of 128 with G/128 a power
  *                   of two, S in {2,3,4,6,8}: plane sums on the matrix cores over
  *                   the raw bit planes, the fp16 activations represented exactly;
- *                   within 2 fp16 ulps of the exact sum.  Taken for M <= 8 always,
- *                   and for 9..16 rows unless the 32-row kernel is preferred;
- *   32-row kernel   5 <= M <= 32, K and G multiples of 32, same S: preferred for
- *                   17..32 rows, for 5..16 rows of shapes the decode kernel has no
- *                   instance for, and for 9..16 rows when N gives at least one
- *                   32-column workgroup per CU of the device (ceil(N/32) >= CUs;
- *                   N >= 8192 on an MI355X);
+ *                   within 2 fp16 ulps of the exact sum.  Taken for every M <= 16
+ *                   of such a shape (5..16 rows in a variant whose waves share the
+ *                   activation operands, where N >= 32 for up to 8 rows, 64 beyond);
+ *   32-row kernel   5 <= M <= 32, K and G multiples of 32, same S: taken for
+ *                   17..32 rows, and for 5..16 rows of shapes the decode kernel
+ *                   does not cover (N < 16, K or G not a multiple of 128);
  *   prefill kernel  M > 32 (or 17..32 with flags bit 1), K and G multiples of 64,
  *                   same S; with a workspace and few output tiles, K is split
  *                   across workgroups;

@@ -39,6 +39,7 @@
 //
 // Portable kernels (any shape, one thread per output) back all of them.
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <mutex>
 #include <stdarg.h>
 #include <stdint.h>
@@ -245,6 +246,28 @@ __device__ __forceinline__ Planes<S> load_planes(const uint32_t *p)
     return r;
 }
 
+// The S fp16 coefficients of table line p as (S + 1) / 2 dwords, in as few loads as the line's alignment allows.
+template <int S>
+__device__ __forceinline__ void load_line_words(const uint16_t *p, uint32_t (&c)[(S + 1) / 2])
+{
+    constexpr int CW = (S + 1) / 2;
+    if constexpr (S == 4) {
+        const uint2 t = *reinterpret_cast<const uint2 *>(p);
+        c[0] = t.x; c[1] = t.y;
+    } else if constexpr (S == 8) {
+        const uint4 t = *reinterpret_cast<const uint4 *>(p);
+        c[0] = t.x; c[1] = t.y; c[2] = t.z; c[3] = t.w;
+    } else if constexpr (S % 2 == 0) {
+#pragma unroll
+        for (int j = 0; j < CW; ++j)
+            c[j] = reinterpret_cast<const uint32_t *>(p)[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < CW; ++j)
+            c[j] = static_cast<uint32_t>(p[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(p[2 * j + 1]) << 16 : 0u);
+    }
+}
+
 // Waves per SIMD the register allocator is asked to leave room for: the A operands and the activations
 // they are made from, the results, the MFMA outputs and plane sums of a unit, the plane words in flight
 // and working registers.
@@ -256,10 +279,11 @@ constexpr int gemv_waves(int S, int MT, int CT, int SP)
 }
 
 // Waves of a workgroup at most: 16, or 8 for the instances that want more than 128 registers a lane
-// (four row tiles, or 8 and more column tiles).
+// (four row tiles).
 constexpr int gemv_max_waves(int MT, int CT)
 {
-    return MT == 4 || CT > 4 ? 8 : kMaxWaves;
+    (void)CT;
+    return MT == 4 ? 8 : kMaxWaves;
 }
 
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
@@ -487,10 +511,7 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     // units at once would sit in the issue of its loads for microseconds (the youngest waves until the launch
     // is nearly over) and make its operands only after that.
     // (workgroups of at most 8 waves keep twice as many, for the same number of requests per CU)
-#ifndef SBVR_AHEAD_WIDE
-#define SBVR_AHEAD_WIDE 6
-#endif
-    constexpr int kAhead = MT > 1 && CT > 4 ? SBVR_AHEAD_WIDE : (gemv_max_waves(MT, CT) == 8 ? 2 * kUnitsAhead : kUnitsAhead);
+    constexpr int kAhead = gemv_max_waves(MT, CT) == 8 ? 2 * kUnitsAhead : kUnitsAhead;
     constexpr int kPre = U < kAhead ? U : kAhead;
     request_units(0, kPre);
     __builtin_amdgcn_sched_barrier(0);       // these requests are out before anything waits
@@ -621,22 +642,7 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
         for (int iw = 0; iw < IW; ++iw) {
             const uint32_t line = static_cast<uint32_t>(min(lraw[sgi][iw], a.L - 1));
-            const uint16_t *p = a.cache + line * S;
-            if constexpr (S == 4) {
-                const uint2 t = *reinterpret_cast<const uint2 *>(p);
-                cl[sgi][iw][0] = t.x; cl[sgi][iw][1] = t.y;
-            } else if constexpr (S == 8) {
-                const uint4 t = *reinterpret_cast<const uint4 *>(p);
-                cl[sgi][iw][0] = t.x; cl[sgi][iw][1] = t.y; cl[sgi][iw][2] = t.z; cl[sgi][iw][3] = t.w;
-            } else if constexpr (S % 2 == 0) {
-#pragma unroll
-                for (int j = 0; j < CW; ++j)
-                    cl[sgi][iw][j] = reinterpret_cast<const uint32_t *>(p)[j];
-            } else {
-#pragma unroll
-                for (int j = 0; j < CW; ++j)
-                    cl[sgi][iw][j] = static_cast<uint32_t>(p[2 * j]) | (2 * j + 1 < S ? static_cast<uint32_t>(p[2 * j + 1]) << 16 : 0u);
-            }
+            load_line_words<S>(a.cache + line * S, cl[sgi][iw]);
         }
     SBVR_STAMP(3);
 
@@ -772,6 +778,253 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     SBVR_STAMP(6);
 }
 
+// 5..16 batch rows (MT = 2 or 4 row tiles of 4).  Per row and sub-group the A operands cost some 30 VALU
+// instructions, as much as a unit's own arithmetic, so here MT waves share the operands of a sub-group: wave
+// (group g, role r) of a workgroup makes row tile r of the group's SP sub-groups (into LDS, where the byte
+// transpose happens anyway), and after one barrier reads all MT tiles back and takes CTW of the group's
+// CTW * MT column tiles.  A workgroup owns 16 * CTW * MT columns and waves / MT sub-group sets; everything
+// else (requests a few units ahead, edge windows, LDS reduction, split-K accumulators) is as in the kernel
+// above.  The MFMAs of a unit go two planes at a time, so that four row tiles fit 128 registers.
+template <int S, int MT, int CTW, int SP>
+__global__ void __launch_bounds__(64 * kMaxWaves)
+sbvr_gemv_batch_kernel(const GemvArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    static_assert(MT == 2 || MT == 4, "two or four row tiles");
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int waves = static_cast<int>(blockDim.x >> 6);
+    const int groups = waves / MT;
+    const int grp = wave / MT, role = wave % MT;
+    const int N = a.N;
+    const int col = lane & 15;   // column inside a tile (B and D operands)
+    const int blk = lane >> 4;   // word of the sub-group (B), batch row of the tile (D)
+    const int sg0 = (blockIdx.y * groups + grp) * SP;     // first sub-group of this wave's group
+    constexpr int W = CTW * MT * 16;                      // columns of the workgroup's window
+    const int bx = gridDim.x % 8 == 0 ? static_cast<int>((blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8)
+                                      : static_cast<int>(blockIdx.x);
+    const int n_own = bx * a.wstride;
+    const int n_base = min(n_own, N - W);
+    const int w_lim = n_base == n_own ? a.wstride : W;    // (columns of the window that are this workgroup's to load)
+    const int ws = role * CTW * 16;                       // this wave's columns of the window start here
+    unsigned char *const images = smem;                                                    // [group][sub-group][row tile] 2 KiB
+    float *const scl = reinterpret_cast<float *>(smem + waves * SP * 2048);                // [group][sub-group][row tile][row]
+    float *const red = reinterpret_cast<float *>(smem + waves * SP * (2048 + 16));         // [wave][tile][row tile][lane]
+
+    SBVR_STAMP(0);
+    // -- 1. requests
+    constexpr int U = SP * CTW;
+    uint32_t xx[SP][4];
+#pragma unroll
+    for (int sgi = 0; sgi < SP; ++sgi)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            xx[sgi][r] = 0u;
+            if (role * 4 + r < a.M) {        // wave-uniform
+                const size_t at = static_cast<size_t>(role * 4 + r) * a.xstride + static_cast<size_t>(sg0 + sgi) * kSub;
+                xx[sgi][r] = reinterpret_cast<const uint32_t *>(a.x + at)[lane];
+            }
+        }
+    constexpr int IW = (16 * CTW + 63) / 64;
+    int lraw[SP][IW];
+#pragma unroll
+    for (int iw = 0; iw < IW; ++iw) {
+        const uint32_t lane_i = static_cast<uint32_t>(n_base + ws + min(64 * iw + lane, 16 * CTW - 1));
+        if (a.idx16) {
+#pragma unroll
+            for (int sgi = 0; sgi < SP; ++sgi)
+                lraw[sgi][iw] = static_cast<const uint16_t *>(a.idx)[static_cast<size_t>((sg0 + sgi) >> a.gshift) * N + lane_i];
+        } else {
+#pragma unroll
+            for (int sgi = 0; sgi < SP; ++sgi)
+                lraw[sgi][iw] = static_cast<const uint8_t *>(a.idx)[static_cast<size_t>((sg0 + sgi) >> a.gshift) * N + lane_i];
+        }
+    }
+    Planes<S> q[U];
+    auto request_units = [&](int u0, int u1) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u >= u0 && u < u1) {
+                const uint32_t *wrow = a.bvr + static_cast<size_t>(sg0 + u / CTW) * 4 * N * S;     // wave-uniform
+                // (columns past the workgroup's own repeat its last one: same cache line, results dropped)
+                const int wc = min(ws + (u % CTW) * 16 + col, w_lim - 1);
+                q[u] = load_planes<S, true>(wrow + (static_cast<uint32_t>(blk) * N + n_base + wc) * S);
+            }
+    };
+    constexpr int kPre = U < kUnitsAhead ? U : kUnitsAhead;
+    request_units(0, kPre);
+    __builtin_amdgcn_sched_barrier(0);
+    SBVR_STAMP(1);
+
+    // -- 2. this wave's row tile of the group's A operands
+    const int off = a_image_byte_offset(8 * (lane >> 2) + (lane & 3), 0);
+    const uint32_t half_sel = (lane & 1) ? 0x07060302u : 0x05040100u;
+    const int fac_log2 = (lane & 3) == 0 ? 2 : ((lane & 3) == 1 ? 1 : 0);
+    __builtin_amdgcn_s_setprio(3);
+#pragma unroll
+    for (int sgi = 0; sgi < SP; ++sgi) {
+        const int slot = (grp * SP + sgi) * MT + role;
+        unsigned char *const img = images + slot * 2048;
+        reinterpret_cast<uint4 *>(img)[lane * 2] = uint4{0u, 0u, 0u, 0u};
+        reinterpret_cast<uint4 *>(img)[lane * 2 + 1] = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float row_scale = 0.f;
+            if (role * 4 + r < a.M) {      // wave-uniform
+                const uint32_t v = xx[sgi][r];
+                const uint32_t amax = wave_umax(max(v & 0x7fffu, (v >> 16) & 0x7fffu));
+                const int eh = min(max(static_cast<int>(amax >> 10), 1), 30);
+                const int e = 20 - eh;
+                row_scale = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
+                const int va = __builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x50, 0xF, 0xF, true);   // quad_perm 0,0,1,1
+                const int vb = __builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xFA, 0xF, 0xF, true);   // quad_perm 2,2,3,3
+                v2h z = as_v2h(__builtin_amdgcn_perm(static_cast<uint32_t>(vb), static_cast<uint32_t>(va), half_sel));
+                const float sc = __uint_as_float(static_cast<uint32_t>(127 - e - fac_log2) << 23);
+                const float sc_last = __uint_as_float(static_cast<uint32_t>(127 - 8 - e - fac_log2) << 23);
+                v2s b = {0, 0};
+                b = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(b, z, sc, false);
+                z -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(as_int(b), sc, false);
+                b = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(b, z, sc, true);
+                z -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(as_int(b), sc, true);
+                const v2s b3 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(v2s{0, 0}, z, sc_last, false);
+                *reinterpret_cast<short *>(img + off + (r * 4 + 0) * 32) = b[0];
+                *reinterpret_cast<short *>(img + off + (r * 4 + 1) * 32) = b[1];
+                *reinterpret_cast<short *>(img + off + (r * 4 + 2) * 32) = b3[0];
+            }
+            if (lane == 0)
+                scl[slot * 4 + r] = row_scale;
+        }
+    }
+    __builtin_amdgcn_s_setprio(0);
+    SBVR_STAMP(7);
+    __syncthreads();
+    SBVR_STAMP(2);
+
+    // -- 3. coefficient lines: lane l gathers the line of this wave's column l (+ 64 iw) for each sub-group
+    constexpr int CW = (S + 1) / 2;
+    uint32_t cl[SP][IW][CW];
+#pragma unroll
+    for (int sgi = 0; sgi < SP; ++sgi)
+#pragma unroll
+        for (int iw = 0; iw < IW; ++iw) {
+            const uint32_t line = static_cast<uint32_t>(min(lraw[sgi][iw], a.L - 1));
+            load_line_words<S>(a.cache + line * S, cl[sgi][iw]);
+        }
+
+    SBVR_STAMP(3);
+    // -- 4. the units
+    float y[CTW][MT];
+#pragma unroll
+    for (int t = 0; t < CTW; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            y[t][mt] = 0.f;
+#pragma unroll
+    for (int sgi = 0; sgi < SP; ++sgi) {
+        v8i A[MT];
+        float scale[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int slot = (grp * SP + sgi) * MT + mt;
+            A[mt] = *reinterpret_cast<const v8i *>(images + slot * 2048 + lane * 32);
+            scale[mt] = scl[slot * 4 + blk];
+        }
+#pragma unroll
+        for (int t = 0; t < CTW; ++t) {
+            const int u = sgi * CTW + t;
+            request_units(u + kPre, u + kPre + 1);
+            float c[S];
+            {
+                uint32_t cqu[CW];
+#pragma unroll
+                for (int j = 0; j < CW; ++j)
+                    cqu[j] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(((t * 16 + col) & 63) * 4,
+                                                                                  static_cast<int>(cl[sgi][(t * 16) / 64][j])));
+#pragma unroll
+                for (int j = 0; j < S; ++j)
+                    c[j] = h2f(static_cast<uint16_t>(j & 1 ? cqu[j / 2] >> 16 : cqu[j / 2] & 0xffffu));
+            }
+            float acc[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                acc[mt] = 0.f;
+#pragma unroll
+            for (int j0 = 0; j0 < S; j0 += 2) {
+                v4f D[MT][2];
+#pragma unroll
+                for (int j = j0; j < S && j < j0 + 2; ++j) {
+                    const uint32_t w = q[u].w[j];
+                    v8i B;
+                    B[0] = static_cast<int>(w & 0x11111111u);
+                    B[1] = static_cast<int>(w & 0x22222222u);
+                    B[2] = static_cast<int>(w & 0x44444444u);
+                    B[3] = static_cast<int>((w >> 1) & 0x44444444u);
+                    B[4] = 0; B[5] = 0; B[6] = 0; B[7] = 0;
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        const v4f z = {0.f, 0.f, 0.f, 0.f};
+                        D[mt][j - j0] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[mt], B, z, 0, 4, 0, 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int j = j0; j < S && j < j0 + 2; ++j)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[mt] = fmaf(c[j], fmaf(D[mt][j - j0][2], 1.f / kLastTermScale, D[mt][j - j0][0] + D[mt][j - j0][1]), acc[mt]);
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                y[t][mt] = fmaf(acc[mt], scale[mt], y[t][mt]);
+        }
+    }
+
+    SBVR_STAMP(4);
+    // -- 5. partial results meet in LDS; summed over the groups in a fixed order
+    constexpr int kBlocks = CTW * MT;                 // (tile, row tile) blocks of a wave
+#pragma unroll
+    for (int t = 0; t < CTW; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            red[(wave * kBlocks + t * MT + mt) * 64 + lane] = y[t][mt];
+    __syncthreads();
+    SBVR_STAMP(5);
+
+    const bool shifted = n_base != n_own;            // window moved left at the edge of N
+    for (int o = wave; o < kBlocks * MT; o += waves) {    // wave-uniform
+        const int role_o = o / kBlocks, rest = o % kBlocks;
+        const int t = rest / MT, mt = rest % MT;
+        float total = 0.f;
+        for (int g = 0; g < groups; ++g)
+            total += red[((g * MT + role_o) * kBlocks + rest) * 64 + lane];
+        const int n = n_base + (role_o * CTW + t) * 16 + col, m = mt * 4 + blk;
+        const bool valid = m < a.M && (!shifted || n >= n_own) && n < n_own + a.wstride;
+        const size_t at = static_cast<size_t>(m) * N + n;
+        if (a.ksplit > 1) {
+            unsigned long long tot = (1ull << 56) + static_cast<unsigned long long>(to_fixed(total) + kAccBias);
+            unsigned long long old = 0ull;
+            if (valid)
+                old = __hip_atomic_fetch_add(a.acc + at, tot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            tot += old;
+            if (!valid || static_cast<int>(tot >> 56) != a.ksplit)
+                continue;
+            const long long sum = static_cast<long long>(tot & ((1ull << 56) - 1)) - (static_cast<long long>(a.ksplit) << 47);
+            const float hi = static_cast<float>(static_cast<int>(sum >> 24));
+            const float lo = static_cast<float>(static_cast<int>(sum & 0xffffff));
+            total = fmaf(hi, 1.f / (1 << (kAccFracBits - 24)), lo * (1.f / (1 << kAccFracBits)));
+            __hip_atomic_store(a.acc + at, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (!valid) {
+            continue;
+        }
+        uint16_t r = f2h(total);
+        if (a.bias)
+            r = hadd(r, a.bias[n]);
+        a.out[at] = r;
+    }
+    SBVR_STAMP(6);
+}
+
 // Launch shape for the MFMA kernel.
 struct GemvPlan {
     int CT, SP, MT, waves, n_wgs, ksplit;
@@ -797,21 +1050,15 @@ const EnvSwitches &env_switches()
     return e;
 }
 
-// (CT, SP) pairs that have a kernel instance; see the dispatch below.  The wide ones (8 column tiles and
-// more) exist for 5..16 batch rows only: there every batch row of a sub-group costs a wave that uses it
-// some 55 VALU instructions of operand preparation, so a wave should use its operands for many columns.
-constexpr int kShapes[][2] = {{1, 1}, {1, 2}, {1, 4}, {1, 7}, {2, 1}, {2, 2}, {2, 4}, {2, 7}, {4, 1}, {4, 2}, {4, 4},
-                              {8, 1}, {8, 2}, {14, 1}, {16, 1}};
+// (CT, SP) pairs that have a kernel instance; see the dispatch below.
+constexpr int kShapes[][2] = {{1, 1}, {1, 2}, {1, 4}, {1, 7}, {2, 1}, {2, 2}, {2, 4}, {2, 7}, {4, 1}, {4, 2}, {4, 4}};
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
 
 constexpr bool shape_ok_for(int MT, int CT, int SP)
 {
-    if (CT > 4)             // registers: A operands 8 * SP * MT, results CT * MT
-        return MT > 1 && SP * MT <= 8 && CT * MT <= 64;
     // (the partial results of a wave, CT*MT*64 floats, fit its 2 KiB buffer up to CT*MT = 8 and get room
-    // of their own beyond)
-    // (two row tiles with a 16-wave launch bound, 128 registers: at most 4 sub-groups of operands, and 4 only
-    // with one column tile)
+    // of their own beyond; two row tiles with a 16-wave launch bound, 128 registers: at most 4 sub-groups
+    // of operands, and 4 only with one column tile)
     return CT * MT <= 16 && (MT == 1 || CT * SP * MT <= 16) && (MT != 2 || (SP <= 4 && CT * SP <= 8 && !(SP == 4 && CT > 1)));
 }
 
@@ -844,36 +1091,6 @@ GemvPlan plan_gemv_uncached(int M, int N, int K, int S, int cus, int min_waves)
     const EnvSwitches &env = env_switches();
     const int eCT = env.ct, eSP = env.sp, eW = env.waves;
     GemvPlan best{};
-    if (MT > 1 && eCT <= 0) {
-        // 5..16 batch rows: a wave's time is its operand preparation (55 VALU instructions per batch row and
-        // sub-group) plus its units (20 + 13 per row tile, and four MFMAs of 32 clocks per row tile, about half
-        // of which hide behind the VALU work): the shape with the smallest estimate of the busiest SIMD's time,
-        // workgroups of up to 8 waves for the wide shapes (they hold up to 256 registers a lane).
-        double best_t = 1e30;
-        for (int i = 0; i < kNumShapes; ++i) {
-            const int CT = kShapes[i][0], SP = kShapes[i][1];
-            if (nsub % SP || !shape_ok_for(MT, CT, SP) || CT * 16 > N)
-                continue;
-            const int parts = nsub / SP;
-            const int windows = (tiles16 + CT - 1) / CT;
-            const int wave_cap = gemv_max_waves(MT, CT);
-            for (int waves = 1; waves <= wave_cap; ++waves) {
-                if (parts % waves || parts / waves > kMaxKsplit)
-                    continue;
-                const int ksplit = parts / waves;
-                const long wgs = static_cast<long>(windows) * ksplit;
-                const long rounds = (wgs + cus - 1) / cus;                       // workgroups the busiest CU runs
-                const double per_wave = 55.0 * SP * M + static_cast<double>(CT) * SP * (20.0 + 13.0 * MT + 16.0 * MT);
-                double t = static_cast<double>(rounds) * ((waves + 3) / 4) * per_wave;
-                t += 0.02 * static_cast<double>(M) * N * ksplit / cus;          // the accumulators' atomics
-                t *= static_cast<double>(windows) * CT / tiles16;               // columns computed for nothing at the edge
-                if (t < best_t) {
-                    best_t = t;
-                    best = GemvPlan{CT, SP, MT, waves, windows, ksplit, 0, CT * 16};
-                }
-            }
-        }
-    }
     // (with the add + norm prologue the waves of a workgroup meet at a barrier before their operands: 8-wave
     // workgroups with four sub-groups a wave measured 14.1-14.7 us against 16.0 for 16 waves with two at
     // 4096 -> 28672, and only that large a matrix gains from taking all of K into the workgroup)
@@ -1004,7 +1221,6 @@ hipError_t launch_gemv_shape(const GemvArgs &a, const GemvPlan &p, hipStream_t s
     SBVR_SHAPE(1, 1); SBVR_SHAPE(1, 2); SBVR_SHAPE(1, 4); SBVR_SHAPE(1, 7);
     SBVR_SHAPE(2, 1); SBVR_SHAPE(2, 2); SBVR_SHAPE(2, 4); SBVR_SHAPE(2, 7);
     SBVR_SHAPE(4, 1); SBVR_SHAPE(4, 2); SBVR_SHAPE(4, 4);
-    SBVR_SHAPE(8, 1); SBVR_SHAPE(8, 2); SBVR_SHAPE(14, 1); SBVR_SHAPE(16, 1);
 #undef SBVR_SHAPE
     return hipErrorInvalidConfiguration;
 }
@@ -1037,6 +1253,147 @@ hipError_t launch_gemv(int S, const GemvArgs &a, const GemvPlan &p, int xm, hipS
     case 3: return launch_gemv_mt<3>(a, p, xm, st);
     case 6: return launch_gemv_mt<6>(a, p, xm, st);
     case 8: return launch_gemv_mt<8>(a, p, xm, st);
+#endif
+    default: return hipErrorInvalidConfiguration;
+    }
+}
+
+// ---- launch shape and dispatch of the kernel for 5..16 batch rows
+struct BatchPlan {
+    int MT, CTW, SP, waves, n_wgs, ksplit, wstride;
+    size_t lds;
+};
+
+constexpr bool batch_shape_ok(int MT, int CTW, int SP)
+{
+    if (SP != 1 && SP != 2 && SP != 4)
+        return false;
+    if (MT == 2)         // (four sub-groups with 7 or 8 tiles, or with 4 tiles x 4 row tiles: more than 128 registers)
+        return CTW == 1 || CTW == 2 || CTW == 4 || ((CTW == 7 || CTW == 8) && SP < 4);
+    return MT == 4 && (CTW == 1 || CTW == 2 || (CTW == 4 && SP < 4));
+}
+
+bool batch_path_ok(int M, int N, int K, int S, int G)
+{
+    return M > 4 && mfma_path_ok(M, N, K, S, G) && N >= 16 * (M <= 8 ? 2 : 4);
+}
+
+// The shape with the smallest estimate of the launch's time: the busiest CU's workgroups one after the
+// other, a workgroup's time that of its waves on one SIMD (operands, then units), plus the accumulators'
+// atomic adds where K is split.
+BatchPlan plan_batch_uncached(int M, int N, int K, int S, int cus)
+{
+    const int nsub = K / kSub;
+    const int MT = M <= 8 ? 2 : 4;
+    const EnvSwitches &env = env_switches();
+    BatchPlan best{};
+    double best_t = 1e30;
+    constexpr int kCtw[] = {1, 2, 4, 7, 8}, kSp[] = {1, 2, 4}, kWaves[] = {16, 8, 4};
+    for (int CTW : kCtw)
+        for (int SP : kSp)
+            for (int waves : kWaves) {
+                if (!batch_shape_ok(MT, CTW, SP) || waves < MT || CTW * MT * 16 > N)
+                    continue;
+                if ((env.ct > 0 && CTW != env.ct) || (env.sp > 0 && SP != env.sp) || (env.waves > 0 && waves != env.waves))
+                    continue;
+                const int groups = waves / MT;
+                if (nsub % (SP * groups) || nsub / (SP * groups) > kMaxKsplit)
+                    continue;
+                const int ksplit = nsub / (SP * groups);
+                const int W = CTW * MT * 16;
+                int windows = (N + W - 1) / W;
+                const int wstride = ((N + windows - 1) / windows + 7) / 8 * 8;
+                windows = (N + wstride - 1) / wstride;
+                const size_t lds = static_cast<size_t>(waves) * (SP * (2048 + 16) + CTW * MT * 256);
+                if (lds > 160 * 1024)
+                    continue;
+                const int per_cu = static_cast<int>(std::min<size_t>(16 / waves, (160 * 1024) / lds));
+                const long wgs = static_cast<long>(windows) * ksplit;
+                const long rounds = (wgs + static_cast<long>(cus) * per_cu - 1) / (static_cast<long>(cus) * per_cu);
+                const double per_wave = SP * (4 * 160.0 + CTW * (MT * S * 32.0 + 250.0)) + CTW * MT * 30.0;
+                double t = 1500.0 + static_cast<double>(rounds) * (waves * per_cu / 4.0) * per_wave;
+                t += 0.05 * static_cast<double>(M) * N * ksplit / cus * (ksplit > 1);
+                t *= static_cast<double>(windows) * W / N;
+                if (t < best_t) {
+                    best_t = t;
+                    best = BatchPlan{MT, CTW, SP, waves, windows, ksplit, wstride, lds};
+                }
+            }
+    return best;
+}
+
+BatchPlan plan_batch(int M, int N, int K, int S, int cus)
+{
+    struct Entry {
+        int M, N, K, S, cus;
+        BatchPlan plan;
+    };
+    constexpr int kEntries = 64;
+    static Entry cache[kEntries];
+    static int used = 0;
+    static std::mutex lock;
+    std::lock_guard<std::mutex> guard(lock);
+    for (int i = 0; i < used; ++i) {
+        const Entry &e = cache[i];
+        if (e.M == M && e.N == N && e.K == K && e.S == S && e.cus == cus)
+            return e.plan;
+    }
+    const BatchPlan p = plan_batch_uncached(M, N, K, S, cus);
+    if (used < kEntries)
+        cache[used++] = Entry{M, N, K, S, cus, p};
+    return p;
+}
+
+template <int S, int MT, int CTW, int SP>
+hipError_t launch_batch_inst(const GemvArgs &a, const BatchPlan &p, hipStream_t st)
+{
+    const dim3 grid(static_cast<unsigned>(p.n_wgs), static_cast<unsigned>(p.ksplit)), block(64 * p.waves);
+    if (p.lds > 65536) {        // above what a kernel gets without asking
+        static bool raised_on[16] = {};
+        int dev_now = 0;
+        if (hipGetDevice(&dev_now) != hipSuccess || dev_now < 0 || dev_now >= 16)
+            dev_now = 0;
+        if (!raised_on[dev_now]) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sbvr_gemv_batch_kernel<S, MT, CTW, SP>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess)
+                return e;
+            raised_on[dev_now] = true;
+        }
+    }
+    hipLaunchKernelGGL((sbvr_gemv_batch_kernel<S, MT, CTW, SP>), grid, block, p.lds, st, a);
+    return hipGetLastError();
+}
+
+template <int S, int MT>
+hipError_t launch_batch_shape(const GemvArgs &a, const BatchPlan &p, hipStream_t st)
+{
+#define SBVR_BSHAPE(ctw, sp)                                \
+    if constexpr (batch_shape_ok(MT, ctw, sp))              \
+        if (p.CTW == ctw && p.SP == sp)                     \
+            return launch_batch_inst<S, MT, ctw, sp>(a, p, st)
+    SBVR_BSHAPE(1, 1); SBVR_BSHAPE(2, 1); SBVR_BSHAPE(4, 1); SBVR_BSHAPE(7, 1); SBVR_BSHAPE(8, 1);
+    SBVR_BSHAPE(1, 2); SBVR_BSHAPE(2, 2); SBVR_BSHAPE(4, 2); SBVR_BSHAPE(7, 2); SBVR_BSHAPE(8, 2);
+    SBVR_BSHAPE(1, 4); SBVR_BSHAPE(2, 4); SBVR_BSHAPE(4, 4); SBVR_BSHAPE(7, 4); SBVR_BSHAPE(8, 4);
+#undef SBVR_BSHAPE
+    return hipErrorInvalidConfiguration;
+}
+
+template <int S>
+hipError_t launch_batch_mt(const GemvArgs &a, const BatchPlan &p, hipStream_t st)
+{
+    return p.MT == 2 ? launch_batch_shape<S, 2>(a, p, st) : launch_batch_shape<S, 4>(a, p, st);
+}
+
+hipError_t launch_batch(int S, const GemvArgs &a, const BatchPlan &p, hipStream_t st)
+{
+    switch (S) {
+    case 4: return launch_batch_mt<4>(a, p, st);
+#ifndef SBVR_FAST_BUILD
+    case 2: return launch_batch_mt<2>(a, p, st);
+    case 3: return launch_batch_mt<3>(a, p, st);
+    case 6: return launch_batch_mt<6>(a, p, st);
+    case 8: return launch_batch_mt<8>(a, p, st);
 #endif
     default: return hipErrorInvalidConfiguration;
     }
@@ -1599,11 +1956,11 @@ bool rows32_path_ok(int M, int N, int K, int S, int G)
 // and 34 us at 16; with fewer than one 32-column workgroup per CU the 32-row kernel loses.
 bool rows32_preferred(int M, int N, int K, int S, int G, int cus)
 {
+    (void)cus;
     if (!rows32_path_ok(M, N, K, S, G))
         return false;
-    if (M <= kMaxM && mfma_path_ok(M, N, K, S, G))
-        return M > 8 && (N + 31) / 32 >= cus;
-    return true;          // no decode kernel for this shape, or 17..32 rows
+    // up to 16 rows the decode kernels are faster wherever they have a shape for (M, N)
+    return !(M <= kMaxM && mfma_path_ok(M, N, K, S, G));
 }
 
 hipError_t launch_rows32(int S, RowsArgs a, hipStream_t st)
@@ -2202,6 +2559,43 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
             return fail(SBVR_HIP_ELAUNCH, "rows32 launch: %s", hipGetErrorString(e));
         g_last_kernel = SBVR_HIP_KERNEL_ROWS32;
         return SBVR_HIP_OK;
+    }
+    if (pro.mode == kXPlain && !(flags & 1) && aligned && batch_path_ok(M, N, K, S, G)) {
+        const BatchPlan p = plan_batch(M, N, K, S, current_cus());
+        if (p.CTW > 0) {
+            if (env_switches().show_plan)
+                fprintf(stderr, "sbvr_hip batch plan M=%d N=%d K=%d S=%d: MT=%d CTW=%d SP=%d waves=%d wgs=%d ksplit=%d wstride=%d lds=%zu\n", M, N, K, S,
+                        p.MT, p.CTW, p.SP, p.waves, p.n_wgs, p.ksplit, p.wstride, p.lds);
+            GemvArgs a{};
+            a.x = static_cast<const uint16_t *>(x);
+            a.bvr = bvr;
+            a.idx = coeff_idx;
+            a.cache = static_cast<const uint16_t *>(coeff_cache);
+            a.bias = static_cast<const uint16_t *>(bias);
+            a.out = static_cast<uint16_t *>(out);
+            a.M = M; a.N = N; a.K = K; a.L = L;
+            a.gshift = __builtin_ctz(static_cast<unsigned>(G / kSub));
+            a.idx16 = idx_bytes == 2;
+            a.ksplit = p.ksplit;
+            a.xstride = K;
+            a.wstride = p.wstride;
+#ifdef SBVR_TRACE
+            a.trace = g_trace;
+#endif
+            if (p.ksplit > 1) {
+                const size_t need = static_cast<size_t>(M) * N * sizeof(unsigned long long);
+                if (!workspace || workspace_bytes < need)
+                    return fail(SBVR_HIP_EWORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+                if (reinterpret_cast<uintptr_t>(workspace) % 8 != 0)
+                    return fail(SBVR_HIP_EINVAL, "workspace must be 8-byte aligned");
+                a.acc = static_cast<unsigned long long *>(workspace);
+            }
+            const hipError_t e = launch_batch(S, a, p, st);
+            if (e != hipSuccess)
+                return fail(SBVR_HIP_ELAUNCH, "batch launch (MT=%d CTW=%d SP=%d waves=%d ksplit=%d): %s", p.MT, p.CTW, p.SP, p.waves, p.ksplit, hipGetErrorString(e));
+            g_last_kernel = SBVR_HIP_KERNEL_DECODE;
+            return SBVR_HIP_OK;
+        }
     }
     if ((!(flags & 1) || pro.mode != kXPlain) && aligned && mfma_path_ok(M, N, K, S, G)) {
         // add + norm: the threads of a workgroup share out all of K, at most kNormChunksMax chunks of 8 each

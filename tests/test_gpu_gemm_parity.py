@@ -89,7 +89,7 @@ def test_rows32_kernel_rows(oracle, M):
 
 @pytest.mark.parametrize("M", [5, 8, 16])
 def test_rows32_kernel_few_rows_short_groups(oracle, M):
-    """5..16 rows reach it where the decode kernel has no instance (groups of 32 or 64)."""
+    """5..16 rows reach it where the decode kernel does not cover the shape (groups of 32 or 64)."""
     run_case(oracle, 256, 512, 4, 64, M, 256, seed=170 + M, expect=ROWS32)
 
 
@@ -112,8 +112,8 @@ def test_rows32_kernel_u16_index_and_bias(oracle):
 
 @pytest.mark.parametrize("S", [2, 3, 4])
 def test_rows32_kernel_gate_shape(oracle, S):
-    """16 rows at 4096 -> 14336: one 32-column workgroup per CU and more, so the default is the 32-row kernel."""
-    run_case(oracle, 14336, 4096, S, 128, 16, 256, seed=97 + S, expect=ROWS32)
+    """17 rows at 4096 -> 14336: the first batch size beyond the decode kernel."""
+    run_case(oracle, 14336, 4096, S, 128, 17, 256, seed=97 + S, expect=ROWS32)
 
 
 def test_matches_decode_path_rows():

@@ -60,9 +60,7 @@ def test_small_m1(oracle, S, G):
 
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 16])
 def test_batch(oracle, M):
-    # flags bit 1 keeps the decode kernel above 4 rows (the default there is the 32-row kernel,
-    # which has its own tests and tolerance in test_gpu_gemm_parity.py)
-    run_case(oracle, 512, 1024, 4, 128, M, 256, seed=3, flags=2 if M > 4 else 0)
+    run_case(oracle, 512, 1024, 4, 128, M, 256, seed=3)
 
 
 def test_u16_index(oracle):
@@ -93,31 +91,85 @@ def test_llama_shapes(oracle, N, K):
 @pytest.mark.parametrize("S", [2, 3, 4])
 @pytest.mark.parametrize("M", [2, 16])
 def test_sweep_gate(oracle, S, M):
-    run_case(oracle, 14336, 4096, S, 128, M, 256, seed=12, flags=2 if M > 4 else 0)
+    run_case(oracle, 14336, 4096, S, 128, M, 256, seed=12)
 
 
 @pytest.mark.parametrize("S", [2, 3, 4])
 @pytest.mark.parametrize("M", [4, 8])
 def test_sweep_down(oracle, S, M):
     """The other shape of the batch / plane sweep: 14336 -> 4096, long K (split across workgroups)."""
-    run_case(oracle, 4096, 14336, S, 128, M, 256, seed=14, flags=2 if M > 4 else 0)
+    run_case(oracle, 4096, 14336, S, 128, M, 256, seed=14)
 
 
-def test_sweep_down_default_path_16_rows(oracle):
-    """16 rows at the down shape without flags: whatever kernel the operator picks, same tolerance."""
+def test_sweep_down_16_rows(oracle):
+    """16 rows at the down shape: four row tiles, K split 14 ways through the accumulators."""
+    run_case(oracle, 4096, 14336, 4, 128, 16, 256, seed=15)
+
+
+@pytest.mark.parametrize("M", [5, 6, 7, 8, 9, 12, 13, 16])
+@pytest.mark.parametrize("N", [32, 48, 64, 100, 1000, 1030])
+def test_batch_rows_ragged_n(oracle, M, N):
+    """5..16 rows: the waves of a workgroup share the activation operands of a sub-group and split its
+    columns.  Windows that end inside a tile, windows moved left at the edge of N, and (N below 64 with more
+    than 8 rows) the shapes that fall back to one wave per sub-group."""
+    from sbvr import hip
+    run_case(oracle, N, 512, 4, 128, M, 64, seed=300 + M + N)
+    assert hip.last_kernel() == 2
+
+
+@pytest.mark.parametrize("S", [2, 3, 6, 8])
+@pytest.mark.parametrize("M", [7, 11])
+def test_batch_rows_planes(oracle, S, M):
+    run_case(oracle, 384, 1024, S, 128, M, 200, seed=320 + S + M)
+
+
+@pytest.mark.parametrize("G", [128, 256, 512])
+@pytest.mark.parametrize("M", [8, 16])
+def test_batch_rows_groups(oracle, G, M):
+    run_case(oracle, 512, 2048, 4, G, M, 256, seed=340 + G + M)
+
+
+def test_batch_rows_u16_index_bias_and_scales(oracle):
+    run_case(oracle, 320, 768, 4, 128, 6, 3000, seed=350)
+    run_case(oracle, 320, 768, 3, 128, 14, 5000, seed=351, bias=True)
+    run_case(oracle, 320, 768, 4, 128, 10, 256, seed=352, xscale=100.0)
+    run_case(oracle, 320, 768, 4, 128, 5, 256, seed=353, xscale=1e-3)
+
+
+def test_batch_rows_of_different_magnitude(oracle):
+    """Each batch row has its own scale per sub-group: a row 2^12 times larger than its neighbours, and a
+    zero row, leave the others exact."""
     import sbvr
     from sbvr import synth
     dev = _dev()
-    N, K, S, M = 4096, 14336, 4, 16
-    bvr, idx, cache = synth.random_encoding(N, K, S, 128, 256, seed=15)
-    x = torch.randn((M, K), generator=torch.Generator().manual_seed(16)).to(torch.float16)
-    y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev), None, bvr_len=128)
-    _, yd = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), 128)
-    got = y.float().cpu().numpy().astype(np.float64)
-    rms = float(np.sqrt(np.mean(yd ** 2)))
-    # (the 32-row kernel decodes the weights to fp16 first: judged against half the RMS for small outputs,
-    # as in test_gpu_gemm_parity.py)
-    assert (np.abs(got - yd) / np.maximum(np.abs(yd), 0.5 * rms)).max() <= 1e-2
+    N, K, S, G, M = 256, 1024, 4, 128, 12
+    bvr, idx, cache = synth.random_encoding(N, K, S, G, 256, seed=360)
+    x = torch.randn((M, K), generator=torch.Generator().manual_seed(361))
+    x[3] *= 4096.0
+    x[5] = 0.0
+    x[9] *= 1e-3
+    x = x.to(torch.float16)
+    y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev), None, bvr_len=G)
+    _, yd = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), G)
+    for m in range(M):           # row by row: each against its own RMS
+        if m == 5:
+            assert float(y[m].float().abs().max()) == 0.0
+        else:
+            check(y[m:m + 1], yd[m:m + 1], f"row {m}")
+
+
+def test_batch_rows_repeatable(oracle):
+    """Split K through the accumulators: the same bits on every call, and the workspace left clean."""
+    import sbvr
+    from sbvr import synth
+    dev = _dev()
+    N, K, M = 1024, 4096, 16
+    bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(N, K, 4, 128, 256, seed=370))
+    x = torch.randn((M, K), generator=torch.Generator().manual_seed(371)).to(torch.float16).to(dev)
+    first = sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, bvr_len=128)
+    for _ in range(5):
+        again = sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, bvr_len=128)
+        assert torch.equal(first, again)
 
 
 def test_portable_kernel(oracle):
