@@ -1,0 +1,28 @@
+/* Encoder search on the GPU (libsbvr_hip.so, gfx950).  Device pointers; the
+ * launch goes to `stream` (a hipStream_t, NULL = default stream).  Return
+ * values: 0 ok, -1 invalid argument, -2 unsupported shape, -3 launch error.
+ */
+#ifndef SBVR_HIP_ENCODER_H
+#define SBVR_HIP_ENCODER_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* mse[b, l] = mean over the G values of group b of min_p (data[b, g] - points[l, p])^2, for `groups`
+ * groups and n candidate lines at once: data (groups, G) fp16, points (n, P) fp16 (the P = 2^S subset
+ * sums of each line, 4-byte aligned), mse (groups, n) fp32.  Difference and square are rounded to fp16
+ * and the minimum is taken there, as the reference's search does in its fp16 compute type
+ * (sbvr/core.py:485-495, _data_diff_min_mse: `(data - candidate_matrix)**2`, `.min(dim=-1)`); the sum
+ * over the group is fp32 in element order, divided by G (the reference: `.to(torch.float32).mean(dim=-1)`,
+ * whose order of summation is torch's).  G <= 4096, groups <= 65535, P a power of two up to 64
+ * (S <= 6).  Replaces the error evaluation inside _search_coeff_bias_space (core.py:530-553), which
+ * the reference runs for one group at a time (core.py:711-722). */
+int sbvr_hip_encoder_group_mse_f16(const void *data, const void *points, float *mse, int groups, int G, int n, int P,
+                                   void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

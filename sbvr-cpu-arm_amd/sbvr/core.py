@@ -227,14 +227,19 @@ class sbvr(torch.nn.Module):
         sel = torch.empty(flat.numel(), dtype=torch.int32, device=data.device)
         if self.verbose_level > 0:
             print(conf.describe())
-        groups = range(n_groups)
+        bar = None
         if self.verbose_level > 0:
             from tqdm import tqdm
-            groups = tqdm(groups, ncols=80, desc="Encoding SBVR groups", unit="g")
-        for i in groups:
-            line, s = enc.encode_group(flat[i * G:(i + 1) * G])
-            line_of[i] = line
-            sel[i * G:(i + 1) * G] = s
+            bar = tqdm(total=n_groups, ncols=80, desc="Encoding SBVR groups", unit="g")
+        # table look-ups for a block of groups at a time on a GPU; the reference's one-group loop on the CPU
+        block = getattr(conf, "group_block", None)
+        if block is None:
+            block = 512 if data.is_cuda else 1
+        line_tmp = torch.empty(n_groups, dtype=torch.int32, device=data.device)
+        enc.encode_all(flat, line_tmp, sel, block=block, progress=bar.update if bar is not None else None)
+        line_of.copy_(line_tmp.to(torch.uint16) if line_of.dtype == torch.uint16 else line_tmp)
+        if bar is not None:
+            bar.close()
         rows = flat.numel() // padded_shape[-1]
         planes = layout.sel_to_planes(sel, self.num_sums, self.bvr_dtype)
         if v1 and rows > 1:

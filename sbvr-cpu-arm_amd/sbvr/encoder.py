@@ -3,10 +3,19 @@ fp16 coefficients whose 2^S subset sums approximate the group best (MSE), and
 reuse earlier lines through a table (the "coefficient cache").
 
 This is the reference's CPU/torch algorithm (sbvr/core.py:19-60 configuration,
-:368-483 search spaces, :485-553 search, :555-653 per-group policy) restated;
-run on the same device with the same configuration it makes the same torch
-calls in the same order, so it yields the same lines and selectors.  It is not
-a GPU kernel and is not on the hot path.
+:368-483 search spaces, :485-553 search, :555-653 per-group policy) restated.
+On the CPU it makes the same torch calls in the same order, so it yields the
+same lines and selectors.  On a GPU two things differ from the reference's loop
+(core.py:711-722, one group at a time):
+  * the error of a (group, line) pair comes from a HIP kernel that keeps the
+    (lines, G, 2^S) tensor of squared differences in registers (hip.encoder_group_mse;
+    fp16 compute type and S <= 6, otherwise the torch expression);
+  * table look-ups run for a block of groups at once (``encode_all``): the
+    groups of a block are looked up against the table as it stands, the leading
+    hits are taken, the first miss goes through the one-group path (which may add
+    a line and move the cut-off), and the look-up restarts behind it.  The policy
+    is order-dependent and this keeps its order: block size 1 and block size 512
+    give the same table, indices and selectors.
 """
 import math
 
@@ -27,7 +36,7 @@ class EncoderConfig:
     )
 
     def __init__(self, **kwargs):
-        unknown = set(kwargs) - set(self.DEFAULTS) - {"bvr_len"}
+        unknown = set(kwargs) - set(self.DEFAULTS) - {"bvr_len", "group_block"}
         if unknown:
             raise TypeError(f"unknown encoder option(s): {sorted(unknown)}")
         for k, v in self.DEFAULTS.items():
@@ -36,6 +45,8 @@ class EncoderConfig:
             self.mse_history = []
         # extension: the reference fixes the group length at 256 (core.py:222)
         self.bvr_len = kwargs.get("bvr_len", 256)
+        # extension: groups looked up in the table at a time (None: 512 on a GPU, 1 on the CPU; see encode_all)
+        self.group_block = kwargs.get("group_block", None)
 
     def describe(self):
         return ("SBVR encoder: num_sums=%d bvr_len=%d r/b/s search=%d/%d/%d window=%d extend=%.2f/%.2f "
@@ -133,10 +144,40 @@ class GroupEncoder:
 
     # -- search ---------------------------------------------------------------
 
+    def _use_kernel(self, data):
+        if not data.is_cuda:
+            return False
+        from . import hip
+        return hip.encoder_group_mse_supported(data.dtype, data.shape[-1], 1 << self.S)
+
+    def _mse_matrix(self, datas, points):
+        """(groups, lines) errors: mean over the group of the squared distance to the nearest point, the
+        differences and squares in the compute type (core.py:485-495)."""
+        if self._use_kernel(datas):
+            from . import hip
+            return hip.encoder_group_mse(datas.contiguous(), points.contiguous())
+        out = torch.empty((datas.shape[0], points.shape[0]), dtype=torch.float32, device=datas.device)
+        # (bounded intermediate: about 2^24 squared differences at a time)
+        step = max(1, (1 << 24) // max(1, points.shape[0] * datas.shape[1] * points.shape[1]))
+        for lo in range(0, datas.shape[0], step):
+            d = datas[lo:lo + step]
+            err = (d.view(d.shape[0], 1, -1, 1) - points.view(1, points.shape[0], 1, points.shape[1])) ** 2
+            out[lo:lo + step] = err.min(dim=-1)[0].to(torch.float32).mean(dim=-1)
+        return out
+
+    def _selectors(self, datas, points):
+        """Nearest point of its own line for every value: datas (groups, G), points (groups, 2^S)."""
+        err = (datas.unsqueeze(-1) - points.unsqueeze(1)) ** 2
+        return err.min(dim=-1)[1]
+
     def _best_in_batch(self, data, lines):
         """MSE of every line's nearest-point quantisation of ``data``; the best
         line and its selectors (core.py:485-501, 521-528)."""
         points = lines @ self.combs.T                                        # (n, 2^S)
+        if self._use_kernel(data):
+            mse = self._mse_matrix(data.view(1, -1), points)[0]
+            at = mse.argmin()
+            return mse[at].item(), at, self._selectors(data.view(1, -1), points[at].view(1, -1))[0]
         err = (data.view(1, -1, 1) - points.view(points.shape[0], 1, points.shape[1])) ** 2
         best_err, best_point = err.min(dim=-1)
         mse = best_err.to(torch.float32).mean(dim=-1)
@@ -168,10 +209,7 @@ class GroupEncoder:
         warming = c.num_coeff_cache_lines < c.cache_warmup_num
         if not warming:
             known = self.table[:c.num_coeff_cache_lines]
-            window = c.mse_history[-min(len(c.mse_history), c.mse_window_size):]
-            cutoff = (sum(window) / len(window)) * 0.99
-            if cutoff < c.acceptable_mse:
-                cutoff = c.acceptable_mse
+            cutoff = self._cutoff()
             best, line_idx, sel = self.search(known, data, cutoff)
             if best < cutoff:
                 c.cache_hits += 1
@@ -192,6 +230,101 @@ class GroupEncoder:
                 sel = new_sel
                 c.mse_history.append(new_mse)
         return line_idx, sel
+
+
+    # -- many groups ----------------------------------------------------------
+
+    def _cutoff(self):
+        c = self.conf
+        window = c.mse_history[-min(len(c.mse_history), c.mse_window_size):]
+        cutoff = (sum(window) / len(window)) * 0.99
+        return c.acceptable_mse if cutoff < c.acceptable_mse else cutoff
+
+    def _lookup_block(self, datas, cutoff):
+        """``search(table, data, cutoff)`` for every row of ``datas`` at once: the same scan over batches
+        of ``search_batch_size`` lines (first strictly better batch winner, stop below the cut-off).
+        Returns python lists (best error, line) per group and the points of every table line (from the
+        same products the scan used)."""
+        c = self.conf
+        n = c.num_coeff_cache_lines
+        known = self.table[:n]
+        step = c.search_batch_size
+        B = datas.shape[0]
+        best = [float("inf")] * B
+        line = [-1] * B
+        live = list(range(B))
+        all_points = []
+        for lo in range(0, n, step):
+            points = known[lo:lo + step] @ self.combs.T
+            all_points.append(points)
+            if not live:
+                continue
+            rows = datas if len(live) == B else datas[torch.tensor(live, device=datas.device)]
+            mse = self._mse_matrix(rows, points)
+            at = mse.argmin(dim=1)
+            val = mse.gather(1, at.view(-1, 1)).view(-1).tolist()
+            at = at.tolist()
+            still = []
+            for j, b in enumerate(live):
+                if val[j] < best[b]:
+                    best[b], line[b] = val[j], lo + at[j]
+                if not best[b] < cutoff:
+                    still.append(b)
+            live = still
+        return best, line, torch.cat(all_points, dim=0)
+
+    def encode_all(self, flat, line_of, sel, block=512, progress=None):
+        """Encodes the groups of ``flat`` (a multiple of bvr_len values) in order into ``line_of`` (one
+        line index per group) and ``sel`` (one selector per value).  ``block`` groups are looked up in the
+        table at a time; 1 is the reference's loop (core.py:711-722)."""
+        c = self.conf
+        G = c.bvr_len
+        n_groups = flat.numel() // G
+        i = 0
+        span = block
+        while i < n_groups:
+            warming = c.num_coeff_cache_lines < c.cache_warmup_num
+            if block <= 1 or warming:
+                line, s = self.encode_group(flat[i * G:(i + 1) * G])
+                line_of[i] = line
+                sel[i * G:(i + 1) * G] = s
+                i += 1
+                if progress is not None:
+                    progress(1)
+                continue
+            B = min(span, n_groups - i)
+            datas = flat[i * G:(i + B) * G].view(B, G)
+            cutoff = self._cutoff()
+            best, line, points = self._lookup_block(datas, cutoff)
+            j = 0
+            restart = False
+            while j < B and not restart:
+                if best[j] < cutoff:
+                    run = j
+                    while run < B and best[run] < cutoff:
+                        run += 1
+                    lines_t = torch.tensor(line[j:run], device=flat.device)
+                    s = self._selectors(datas[j:run], points[lines_t])
+                    line_of[i + j:i + run] = lines_t.to(line_of.dtype)
+                    sel[(i + j) * G:(i + run) * G] = s.reshape(-1)
+                    c.cache_hits += run - j
+                    c.group_idx += run - j
+                    if progress is not None:
+                        progress(run - j)
+                    j = run
+                else:
+                    before = (c.num_coeff_cache_lines, len(c.mse_history))
+                    ln, s = self.encode_group(datas[j])
+                    line_of[i + j] = ln
+                    sel[(i + j) * G:(i + j + 1) * G] = s
+                    if progress is not None:
+                        progress(1)
+                    j += 1
+                    # a new line or a new entry of the error history changes what the later groups see
+                    restart = (c.num_coeff_cache_lines, len(c.mse_history)) != before
+            i += j
+            # (short blocks while the table still grows, long ones once it has settled)
+            span = block if not restart else max(16, min(block, 2 * j))
 
 
 def default_batch_size(conf, dtype, device):

@@ -62,6 +62,7 @@ def _load():
     lib.sbvr_hip_dec_argmax_advance_f16.argtypes = [vp, i, vp, vp, vp, i, vp, vp, i, vp, vp]
     lib.sbvr_hip_dec_head_argmax_f16.argtypes = [vp, vp, vp, ctypes.c_float, vp, i, i, vp, vp, vp, vp, i, vp, vp, i,
                                                  vp, vp, vp]
+    lib.sbvr_hip_encoder_group_mse_f16.argtypes = [vp, vp, vp, i, i, i, i, vp]
     _lib = lib
     return lib
 
@@ -402,3 +403,28 @@ def dec_head_argmax(x, delta, weight, eps, head, logits, token, generated, pos, 
         sin.data_ptr() if rot_now is not None else None, head_dim,
         rot_now.data_ptr() if rot_now is not None else None, workspace.data_ptr(), _stream()), "head_argmax")
     return logits
+
+
+def encoder_group_mse(data, points):
+    """mse[b, l] = mean_g min_p (data[b, g] - points[l, p])^2 in the encoder's arithmetic (fp16 difference
+    and square, fp32 sum in element order): data (groups, G) fp16, points (n, P) fp16 -> (groups, n) fp32.
+    The error evaluation of the reference's search (sbvr/core.py:485-495) for many groups at once."""
+    _want(data, "data", torch.float16, 2)
+    _want(points, "points", torch.float16, 2, data.device)
+    groups, G = data.shape
+    n, P = points.shape
+    out = torch.empty((groups, n), dtype=torch.float32, device=data.device)
+    with torch.cuda.device(data.device):
+        done = 0
+        while done < groups:          # (a launch takes at most 65535 groups)
+            take = min(groups - done, 65535)
+            rc = _load().sbvr_hip_encoder_group_mse_f16(data[done:done + take].data_ptr(), points.data_ptr(),
+                                                        out[done:done + take].data_ptr(), take, G, n, P, _stream())
+            if rc != 0:
+                raise SbvrHipError(f"sbvr_hip_encoder_group_mse_f16: error {rc} (groups={take} G={G} n={n} P={P})")
+            done += take
+    return out
+
+
+def encoder_group_mse_supported(dtype, G, P):
+    return dtype == torch.float16 and G <= 4096 and P in (2, 4, 8, 16, 32, 64)

@@ -37,6 +37,20 @@ def test_encoder_reproduces_reference(golden, name):
         assert _same_bits(obj.decode(), _t(g["decoded"]))
 
 
+@pytest.mark.parametrize("name,block", [(n, 64) for n in CASES] + [("v1_s2", 3), ("default_s3", 5)])
+def test_block_lookup_encoder_reproduces_reference(golden, name, block):
+    """Table look-ups for a block of groups at a time (the GPU's default) keep the order-dependent policy:
+    the same arrays as the reference's one-group loop, for a short and a long block."""
+    import sbvr
+    g = golden(name)
+    obj = sbvr.sbvr(_t(g["data"]), encoder_config={"num_sums": int(g["num_sums"]), "group_block": block},
+                    device=torch.device("cpu"), verbose_level=0, **CASES[name])
+    assert _same_bits(obj.bvr.data, _t(g["bvr"]))
+    assert _same_bits(obj.coeff_idx.data, _t(g["coeff_idx"]))
+    assert _same_bits(obj.coeff_cache.data, _t(g["coeff_cache"]))
+    assert obj.encoder_stats["groups"] == obj.coeff_idx.numel()
+
+
 @pytest.mark.parametrize("name", ["default_s2", "default_s3", "default_s4", "pad_s2", "v2_s2", "v1_row_s2",
                                   "trans_s2", "weights_s4"])
 def test_decode_of_reference_arrays(golden, name):
