@@ -312,13 +312,78 @@ class sbvr(torch.nn.Module):
             self.original_dtype, tuple(self.original_data_shape), tuple(self.coeff_idx.shape),
             tuple(self.coeff_cache.shape)))
 
-    # The reference declares an "online" activation-encoding path and leaves it
-    # empty (core.py:971-1027); the names are kept, the behaviour is explicit.
-    def profile_input(self, input, encoder_config=None):
-        raise NotImplementedError("activation profiling is a stub in the reference (core.py:971-1019)")
+    # -- activations encoded on the fly ------------------------------------------
+    # The reference declares this path and leaves its two run-time methods empty (core.py:1021-1027 return
+    # None): profile_input finds one line of input coefficients per group of K from sample activations
+    # (core.py:971-1019); at run time an activation row is encoded against those lines (every element takes
+    # the nearest subset sum of its group's line, the selector rule of the encoder, core.py:492-494) and
+    # multiplied with the encoded weight by the both-encoded operator (core.py:1029-1039).
 
+    def _get_padded_input_shape(self, input):
+        shape = list(input.shape)
+        shape[-1] = _padded(shape[-1], self.bvr_len)
+        return torch.Size(shape)
+
+    @torch.inference_mode()
+    def profile_input(self, input, encoder_config=None):
+        """One line of ``num_sums`` (default 8) input coefficients per group of K, searched over all sample
+        rows of ``input`` (..., K) at once; kept in ``input_coeff`` (K / bvr_len, num_sums)."""
+        if input.shape[-1] != self.original_data_shape[-1]:
+            raise ValueError("Inner dimension shape of the input does not match the original data shape, expected "
+                             f"{self.original_data_shape[-1]} but got {input.size(-1)}")
+        conf = EncoderConfig(**dict(encoder_config if encoder_config is not None else {"num_sums": 8}))
+        dev = self.bvr.device
+        padded_shape = self._get_padded_input_shape(input)
+        padded = torch.zeros(padded_shape, dtype=self.compute_dtype, device=dev)
+        padded[tuple(slice(0, s) for s in input.shape)] = input.to(dev).to(self.compute_dtype)
+        groups = padded_shape[-1] // self.bvr_len
+        # (all rows' values of one group of K side by side: one search per group of K)
+        per_group = padded.view(-1, groups, self.bvr_len).permute(1, 0, 2).contiguous().view(groups, -1)
+        conf.bvr_len = per_group.shape[1]
+        conf.cache_warmup_num = groups                 # every group gets a line of its own
+        if conf.search_batch_size <= 0:
+            conf.search_batch_size = default_batch_size(conf, self.compute_dtype, dev)
+        enc = GroupEncoder(conf, self.compute_dtype, dev, max_lines=groups, verbose=self.verbose_level)
+        for g in range(groups):
+            before = conf.num_coeff_cache_lines
+            line, _ = enc.encode_group(per_group[g])
+            if conf.num_coeff_cache_lines == before:   # (a line equal to an earlier group's: keep one per group)
+                enc.table[before] = enc.table[int(line)]
+                conf.num_coeff_cache_lines = before + 1
+        self.input_num_sums = conf.num_sums
+        self.input_coeff = torch.nn.Parameter(enc.table[:groups].clone(), requires_grad=False)
+
+    @torch.inference_mode()
+    def _online_tranfrom(self, input):
+        """(the reference's spelling) ``input`` (M, K) -> the arrays of an encoded left operand: bvr
+        (K/32, M, S_in) uint32, coeff_idx (K / bvr_len, M), coeff_cache = the input coefficients."""
+        from . import hip
+        if self.input_coeff is None:
+            raise RuntimeError("profile_input() has not been run: no input coefficients")
+        x = input.reshape(-1, input.shape[-1]).to(self.bvr.device).to(self.compute_dtype)
+        k_pad = _padded(x.shape[1], self.bvr_len)
+        if x.shape[1] != k_pad:
+            x = torch.nn.functional.pad(x, (0, k_pad - x.shape[1]))
+        coeff = self.input_coeff.data
+        points = coeff @ layout.bin_combs(coeff.shape[1], self.compute_dtype, coeff.device).T
+        bvr = hip.online_encode(x.contiguous(), points.contiguous(), self.bvr_len)
+        groups = coeff.shape[0]
+        idx = torch.arange(groups, device=coeff.device).view(-1, 1).expand(groups, x.shape[0])
+        idx = idx.to(torch.uint8 if groups <= 256 else torch.uint16).contiguous()
+        return bvr, idx, coeff
+
+    _online_transform = _online_tranfrom
+
+    @torch.inference_mode()
     def online_mm_T(self, rhs, bias=None):
-        raise NotImplementedError("online_mm_T is a stub in the reference (core.py:1024-1027)")
+        """``rhs`` (M, K) activations, encoded on the fly against the profiled input coefficients, times this
+        encoded weight transposed: (M, N) fp16 through the both-encoded operator."""
+        from . import hip
+        if bias is None:
+            bias = self._get_dummy_bias()
+        l_bvr, l_idx, l_cache = self._online_tranfrom(rhs)
+        return hip._sbvr_mm_T(l_bvr, l_idx, l_cache, self.default_layout(torch.uint32), self.coeff_idx.data,
+                              self.coeff_cache.data, bias)
 
 
 def mm_T(lhs, rhs, bias):

@@ -63,6 +63,7 @@ def _load():
     lib.sbvr_hip_dec_head_argmax_f16.argtypes = [vp, vp, vp, ctypes.c_float, vp, i, i, vp, vp, vp, vp, i, vp, vp, i,
                                                  vp, vp, vp]
     lib.sbvr_hip_encoder_group_mse_f16.argtypes = [vp, vp, vp, i, i, i, i, vp]
+    lib.sbvr_hip_online_encode_f16.argtypes = [vp, vp, vp, i, i, i, i, vp]
     _lib = lib
     return lib
 
@@ -427,4 +428,21 @@ def encoder_group_mse(data, points):
 
 
 def encoder_group_mse_supported(dtype, G, P):
-    return dtype == torch.float16 and G <= 4096 and P in (2, 4, 8, 16, 32, 64)
+    return dtype == torch.float16 and P in (2, 4, 8, 16, 32, 64, 128, 256)
+
+
+def online_encode(x, points, bvr_len):
+    """Activations to bit planes on the fly: x (M, K) fp16 and the 2^S subset sums of every K-group's input
+    coefficients, points (K / bvr_len, 2^S) fp16 -> bvr (K/32, M, S) uint32 in the default layout."""
+    _want(x, "x", torch.float16, 2)
+    _want(points, "points", torch.float16, 2, x.device)
+    M, K = x.shape
+    S = points.shape[1].bit_length() - 1
+    if points.shape[1] != 1 << S or K % bvr_len != 0 or points.shape[0] != K // bvr_len:
+        raise ValueError(f"points must be (K / bvr_len, 2^S), got {tuple(points.shape)} for K={K}, bvr_len={bvr_len}")
+    bvr = torch.empty((K // 32, M, S), dtype=torch.uint32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _load().sbvr_hip_online_encode_f16(x.data_ptr(), points.data_ptr(), bvr.data_ptr(), M, K, bvr_len, S, _stream())
+    if rc != 0:
+        raise SbvrHipError(f"sbvr_hip_online_encode_f16: error {rc} (M={M} K={K} bvr_len={bvr_len} S={S})")
+    return bvr
