@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the gate GEMV as the hardware counters saw them: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy.  A profiler run's figure,
 # not measured by this script: the line names the file it comes from.
-TRAFFIC_FROM_PROFILE_BYTES = 30.59e6
+TRAFFIC_FROM_PROFILE_BYTES = 30.09e6
 TRAFFIC_PROFILE = "profiles/sbvr_gemv_mfma_gate_4096x14336.txt"
 MIN_TIMED_LAUNCHES = 200
 _WEIGHTS = None        # the rotating weight copies on the device (built once per process)

@@ -210,6 +210,8 @@ struct Planes {
 };
 
 typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+typedef uint32_t v3raw __attribute__((ext_vector_type(3)));
+typedef v3raw v3u __attribute__((aligned(4)));          // (as it lies in a row of 3 or 6 plane words)
 
 // The S plane words of one (word of K, column) pair.  kStream: non-temporal loads, for kernels that
 // read every plane word once per launch and are bound by that stream (measured on the decode kernel:
@@ -235,9 +237,14 @@ __device__ __forceinline__ Planes<S> load_planes(const uint32_t *p)
         const v4u v0 = ld4(p), v1 = ld4(p + 4);
         r.w[0] = v0.x; r.w[1] = v0.y; r.w[2] = v0.z; r.w[3] = v0.w;
         r.w[4] = v1.x; r.w[5] = v1.y; r.w[6] = v1.z; r.w[7] = v1.w;
+    } else if constexpr (S == 3) {
+        // (12 bytes in one request: a global load wants dword alignment only)
+        const v3raw v = kStream ? __builtin_nontemporal_load(reinterpret_cast<const v3u *>(p)) : *reinterpret_cast<const v3u *>(p);
+        r.w[0] = v.x; r.w[1] = v.y; r.w[2] = v.z;
     } else if constexpr (S == 6) {
-        const v2u v0 = ld2(p), v1 = ld2(p + 2), v2 = ld2(p + 4);
-        r.w[0] = v0.x; r.w[1] = v0.y; r.w[2] = v1.x; r.w[3] = v1.y; r.w[4] = v2.x; r.w[5] = v2.y;
+        const v3raw v0 = kStream ? __builtin_nontemporal_load(reinterpret_cast<const v3u *>(p)) : *reinterpret_cast<const v3u *>(p);
+        const v3raw v1 = kStream ? __builtin_nontemporal_load(reinterpret_cast<const v3u *>(p + 3)) : *reinterpret_cast<const v3u *>(p + 3);
+        r.w[0] = v0.x; r.w[1] = v0.y; r.w[2] = v0.z; r.w[3] = v1.x; r.w[4] = v1.y; r.w[5] = v1.z;
     } else {
 #pragma unroll
         for (int j = 0; j < S; ++j)
@@ -1264,13 +1271,18 @@ struct BatchPlan {
     size_t lds;
 };
 
-constexpr bool batch_shape_ok(int MT, int CTW, int SP)
+constexpr bool batch_shape_ok(int S, int MT, int CTW, int SP)
 {
     if (SP != 1 && SP != 2 && SP != 4)
         return false;
-    if (MT == 2)         // (four sub-groups with 7 or 8 tiles, or with 4 tiles x 4 row tiles: more than 128 registers)
-        return CTW == 1 || CTW == 2 || CTW == 4 || ((CTW == 7 || CTW == 8) && SP < 4);
-    return MT == 4 && (CTW == 1 || CTW == 2 || (CTW == 4 && SP < 4));
+    // (left out: the shapes that do not fit 128 registers a lane for that plane count)
+    if (MT == 2)
+        return CTW == 1 || CTW == 2 || CTW == 4 || ((CTW == 7 || CTW == 8) && SP < 4 && !(S == 6 && CTW == 8 && SP == 2));
+    if (MT != 4)
+        return false;
+    if ((S == 3 || S == 8) && CTW * SP >= 8)
+        return false;
+    return CTW == 1 || CTW == 2 || (CTW == 4 && SP < 4);
 }
 
 bool batch_path_ok(int M, int N, int K, int S, int G)
@@ -1292,7 +1304,7 @@ BatchPlan plan_batch_uncached(int M, int N, int K, int S, int cus)
     for (int CTW : kCtw)
         for (int SP : kSp)
             for (int waves : kWaves) {
-                if (!batch_shape_ok(MT, CTW, SP) || waves < MT || CTW * MT * 16 > N)
+                if (!batch_shape_ok(S, MT, CTW, SP) || waves < MT || CTW * MT * 16 > N)
                     continue;
                 if ((env.ct > 0 && CTW != env.ct) || (env.sp > 0 && SP != env.sp) || (env.waves > 0 && waves != env.waves))
                     continue;
@@ -1311,8 +1323,11 @@ BatchPlan plan_batch_uncached(int M, int N, int K, int S, int cus)
                 const long wgs = static_cast<long>(windows) * ksplit;
                 const long rounds = (wgs + static_cast<long>(cus) * per_cu - 1) / (static_cast<long>(cus) * per_cu);
                 const double per_wave = SP * (4 * 160.0 + CTW * (MT * S * 32.0 + 250.0)) + CTW * MT * 30.0;
-                double t = 1500.0 + static_cast<double>(rounds) * (waves * per_cu / 4.0) * per_wave;
-                t += 0.05 * static_cast<double>(M) * N * ksplit / cus * (ksplit > 1);
+                // (below three waves per SIMD the waits of a wave are not covered by the others)
+                double t = 1500.0 + static_cast<double>(rounds) * std::max(waves * per_cu / 4.0, 3.0) * per_wave;
+                // (measured: 3.6 us for the 917 504 adds of 16 rows x 14336 columns x 4 parts, whatever the shape; with
+                // two row tiles the sweeps are fitted better by a third of that: more of it hides behind the units)
+                t += ksplit > 1 ? (MT == 4 ? 0.0082 : 0.003) * static_cast<double>(M) * N * ksplit : 0.0;
                 t *= static_cast<double>(windows) * W / N;
                 if (t < best_t) {
                     best_t = t;
@@ -1369,7 +1384,7 @@ template <int S, int MT>
 hipError_t launch_batch_shape(const GemvArgs &a, const BatchPlan &p, hipStream_t st)
 {
 #define SBVR_BSHAPE(ctw, sp)                                \
-    if constexpr (batch_shape_ok(MT, ctw, sp))              \
+    if constexpr (batch_shape_ok(S, MT, ctw, sp))           \
         if (p.CTW == ctw && p.SP == sp)                     \
             return launch_batch_inst<S, MT, ctw, sp>(a, p, st)
     SBVR_BSHAPE(1, 1); SBVR_BSHAPE(2, 1); SBVR_BSHAPE(4, 1); SBVR_BSHAPE(7, 1); SBVR_BSHAPE(8, 1);
