@@ -286,5 +286,6 @@ def test_cpu_port_matches_oracle(oracle):
             oracle.PORT.init_pool(threads)
             got = oracle.PORT.mm_T_v1(lb, li, lc, rv1, ri, rc, G, bias).astype(np.float64)
             oracle.PORT.finalize_pool()
-            # the port rounds every coefficient product to fp16, as the reference does
-            assert np.abs(got - want).max() <= 1e-2 * max(np.abs(want).max(), 1.0)
+            # the port rounds every coefficient product to fp16, as the reference does, and adds in another
+            # order than the oracle: the two fp16 results are at most one fp16 step of the largest output apart
+            assert np.abs(got - want).max() <= 2.0 ** -10 * max(np.abs(want).max(), 1.0)
