@@ -181,6 +181,22 @@ int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_co
                           void *stream);
 
 /*
+ * The same product with room for a split of K across workgroups: a workspace of
+ * sbvr_hip_row_deq_mm_T_workspace(M, N) bytes (M*N 64-bit accumulators, zero-filled once, 8-byte
+ * aligned, left zero by every call; it may be the workspace of sbvr_hip_linear_f16, not used by
+ * two calls at once).  With 4 planes, K a multiple of 128 and groups of 64 columns and more the
+ * plane sums run on the matrix cores, and where the columns alone would leave CUs idle (N = 4096
+ * on an MI355X) the parts of K are summed through the accumulators, in fixed point, so the result
+ * does not depend on their order.  workspace NULL: as sbvr_hip_row_deq_mm_T.  The reference's
+ * operator has no such argument (sbvr_ops.cpp:79-120); its bindings here bring their own.
+ */
+int sbvr_hip_row_deq_mm_T_ws(const void *x, const uint32_t *r_bvr, const void *r_coeff_idx,
+                             int idx_bytes, const void *r_coeff_cache, const void *bias,
+                             void *out, int M, int N, int K, int S, int G, int L,
+                             void *workspace, size_t workspace_bytes, void *stream);
+size_t sbvr_hip_row_deq_mm_T_workspace(int M, int N);
+
+/*
  * Both operands SBVR-encoded (default uint32 layout on both sides):
  *   out[m,n] = f16( sum_g sum_l sum_r popcount_g(L_l & R_r) * a_l * b_r ) (+ bias[n])
  * Replaces launch_cuda_sbvr_mm_T, sbvr/kernels/sbvr_kernel.cu:914-1022, called

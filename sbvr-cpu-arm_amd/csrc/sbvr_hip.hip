@@ -1041,7 +1041,7 @@ struct GemvPlan {
 
 // Development switches, read from the environment once per process.
 struct EnvSwitches {
-    int ct, sp, waves, wstride, show_plan, popc_q;
+    int ct, sp, waves, wstride, show_plan, popc_q, rowdeq_lanes;
 };
 
 const EnvSwitches &env_switches()
@@ -1052,7 +1052,7 @@ const EnvSwitches &env_switches()
             return v && *v ? atoi(v) : 0;
         };
         return EnvSwitches{get("SBVR_HIP_CT"), get("SBVR_HIP_SP"), get("SBVR_HIP_WAVES"), get("SBVR_HIP_WSTRIDE"),
-                           get("SBVR_HIP_SHOW_PLAN"), get("SBVR_HIP_POPC_Q")};
+                           get("SBVR_HIP_SHOW_PLAN"), get("SBVR_HIP_POPC_Q"), get("SBVR_HIP_ROWDEQ_LANES")};
     }();
     return e;
 }
@@ -2217,6 +2217,229 @@ sbvr_row_deq_lanes_kernel(const uint16_t *__restrict__ x, const uint32_t *__rest
     }
 }
 
+// The trans=True product on the matrix cores (4 planes, K a multiple of 128, groups of 64 columns and more).
+// A word of this layout holds one row k of 32 columns, so the bits that an MFMA wants along K lie across rows.
+// The lanes of a wave, each holding one row's word, transpose the four 16 x 16 bit blocks of every 32 rows between
+// them in four exchange stages (two DPP quad permutes, one DPP row rotate, one ds_swizzle; per stage a rotate and a
+// bit-field insert): lane 16q + c then holds column c's bits of rows 16q .. 16q+15 in its low half and column
+// 16 + c's in its high half.  Two such loads (rows 0-63 and 64-127 of a sub-group) give the B operands of the word's
+// two column tiles without moving anything between lanes: the low halves of both, side by side, are tile 0's
+// operand (lane group q of an MFMA operand is lanes 16q .. 16q+15: rows 16q .. 16q+15 and 64+16q .. 64+16q+15 of
+// column c), the high halves tile 1's; the A image's bytes are laid out in that order of K.
+// The A operand carries z_j[k] = fp16(x[k] * c_j(line of the column group at row k)) for the four planes as its
+// "batch rows" (plane j: rows 4j .. 4j+2, three exact fp8 terms as in the decode kernel), and the four MFMAs of a
+// unit each use a copy with the other planes' rows zeroed, so they accumulate into one result: lane group j keeps
+// plane j's sum.  A workgroup owns 64 columns of one coefficient group and one batch row; its waves take the
+// sub-groups of K in turn (one A image serves all the workgroup's columns).
+// Numerics: z is rounded to fp16 once (2^-12 relative per product, random sign), everything after that is exact up
+// to the fp32 sums; the one-lane-per-row kernel above keeps z in fp32.
+__device__ __forceinline__ uint32_t transpose_16x16_blocks_across_lanes(uint32_t w, int lane)
+{
+    const int r = lane & 15;
+#define SBVR_TSTAGE(s, Ms, EXCH)                                                             \
+    {                                                                                         \
+        const uint32_t p = EXCH;                                                              \
+        const uint32_t rot = __builtin_amdgcn_alignbit(p, p, (r & s) ? s : 32 - s);           \
+        const uint32_t keep = (r & s) ? Ms : ~Ms;                                             \
+        w = (w & keep) | (rot & ~keep);                                                       \
+    }
+    SBVR_TSTAGE(8, 0xFF00FF00u, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(w), 0x128, 0xF, 0xF, true)))   // row_ror 8
+    SBVR_TSTAGE(4, 0xF0F0F0F0u, static_cast<uint32_t>(__builtin_amdgcn_ds_swizzle(static_cast<int>(w), (4 << 10) | 0x1f)))
+    SBVR_TSTAGE(2, 0xCCCCCCCCu, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(w), 0x4E, 0xF, 0xF, true)))    // quad_perm 2,3,0,1
+    SBVR_TSTAGE(1, 0xAAAAAAAAu, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(w), 0xB1, 0xF, 0xF, true)))    // quad_perm 1,0,3,2
+#undef SBVR_TSTAGE
+    return w;
+}
+
+template <int NWW>
+__global__ void __launch_bounds__(64 * kRowDeqWaves)
+sbvr_row_deq_mfma_kernel(const uint16_t *__restrict__ x, const uint32_t *__restrict__ bvr,
+                         const void *__restrict__ idx, const uint16_t *__restrict__ cache,
+                         const uint16_t *__restrict__ bias, uint16_t *__restrict__ out, unsigned long long *__restrict__ acc_words,
+                         int M, int N, int K, int L, int G, int idx16, int ksplit)
+{
+    constexpr int S = 4;
+    __shared__ __align__(16) unsigned char images[kRowDeqWaves][2048];
+    __shared__ float red[kRowDeqWaves][2 * NWW][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = static_cast<int>(blockDim.x >> 6);
+    const int col = lane & 15, blk = lane >> 4;
+    const int m = blockIdx.y;
+    const int nwords = N / 32;
+    const int nw0 = NWW * blockIdx.x;                     // the workgroup's NWW column words (the last ones may be missing)
+    const int nsub = K / kSub;
+    const size_t ibase = static_cast<size_t>((nw0 * 32) / G) * K;
+    const uint16_t *xrow = x + static_cast<size_t>(m) * K;
+    unsigned char *const img = images[wave];
+
+    // where this lane's two elements (rows 8g + t and 8g + t + 4 of the sub-group, see the decode kernel) sit in the A
+    // image: row k = 64 b + 16 q + i is bit 16 b + i of lane group q's B words
+    const int el = 8 * (lane >> 2) + (lane & 3);
+    const int off = a_image_byte_offset(32 * ((el >> 4) & 3) + 16 * (el >> 6) + (el & 15), 0);
+    const uint32_t half_sel = (lane & 1) ? 0x07060302u : 0x05040100u;
+    const int fac_log2 = (lane & 3) == 0 ? 2 : ((lane & 3) == 1 ? 1 : 0);
+    const int row_plane = (lane & 15) >> 2;               // plane whose terms this lane's A row carries
+
+    // (K split across workgroups, blockIdx.z, where the columns alone leave CUs idle: the parts meet in the 64-bit
+    // fixed-point accumulators of the decode kernel)
+    const int per_part = (nsub + ksplit - 1) / ksplit;
+    const int sg_begin = static_cast<int>(blockIdx.z) * per_part, sg_end = min(nsub, sg_begin + per_part);
+    float acc[NWW][2];
+#pragma unroll
+    for (int h = 0; h < NWW; ++h)
+        acc[h][0] = acc[h][1] = 0.f;
+    // The coefficient lines of a sub-group are two round trips away (line index, then the gather): both are sent for
+    // one sub-group ahead, the indices at the top of the step before, the gathers at its end.
+    auto load_x_idx = [&](int sg, uint32_t &xv, uint32_t &raw) __attribute__((always_inline)) {
+        const int k0 = sg * kSub;
+        xv = reinterpret_cast<const uint32_t *>(xrow + k0)[lane];
+        if (idx16)
+            raw = reinterpret_cast<const uint32_t *>(static_cast<const uint16_t *>(idx) + ibase + k0)[lane];
+        else
+            raw = reinterpret_cast<const uint16_t *>(static_cast<const uint8_t *>(idx) + ibase + k0)[lane];
+    };
+    auto gather_lines = [&](uint32_t raw, uint32_t (&c0)[2], uint32_t (&c1)[2]) __attribute__((always_inline)) {
+        const int l0 = static_cast<int>(idx16 ? raw & 0xffffu : raw & 0xffu), l1 = static_cast<int>(idx16 ? raw >> 16 : (raw >> 8) & 0xffu);
+        load_line_words<S>(cache + static_cast<size_t>(min(l0, L - 1)) * S, c0);
+        load_line_words<S>(cache + static_cast<size_t>(min(l1, L - 1)) * S, c1);
+    };
+    uint32_t xv = 0u, x_next = 0u, raw_next = 0u;
+    uint32_t c0[2] = {0u, 0u}, c1[2] = {0u, 0u}, n0[2] = {0u, 0u}, n1[2] = {0u, 0u};
+    if (sg_begin + wave < sg_end) {
+        uint32_t raw_first;
+        load_x_idx(sg_begin + wave, x_next, raw_first);
+        gather_lines(raw_first, n0, n1);
+    }
+    for (int sg = sg_begin + wave; sg < sg_end; sg += waves) {          // wave-uniform
+        const int k0 = sg * kSub;
+        // -- requests: plane words of the column words (rows k0 .. k0+63 and k0+64 .. k0+127); activations and line
+        //    indices of the next sub-group
+        // (asking for the next sub-group's plane words here as well measured slower: 16.9 against 15.3 us)
+        v4u wa[NWW], wb[NWW];
+#pragma unroll
+        for (int h = 0; h < NWW; ++h) {
+            const uint32_t *base = bvr + static_cast<size_t>(min(nw0 + h, nwords - 1)) * K * S;
+            wa[h] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(base + static_cast<size_t>(k0 + lane) * S));
+            wb[h] = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(base + static_cast<size_t>(k0 + 64 + lane) * S));
+        }
+        xv = x_next;
+        c0[0] = n0[0]; c0[1] = n0[1]; c1[0] = n1[0]; c1[1] = n1[1];
+        const bool more = sg + waves < sg_end;
+        if (more)
+            load_x_idx(sg + waves, x_next, raw_next);
+
+        // -- A image: plane j's row is z_j = fp16(x * c_j) of the 128 rows
+        const float x0 = h2f(static_cast<uint16_t>(xv & 0xffffu)), x1 = h2f(static_cast<uint16_t>(xv >> 16));
+        reinterpret_cast<uint4 *>(img)[lane * 2] = uint4{0u, 0u, 0u, 0u};
+        reinterpret_cast<uint4 *>(img)[lane * 2 + 1] = uint4{0u, 0u, 0u, 0u};
+        float scale_mine = 0.f;
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            const float cj0 = h2f(static_cast<uint16_t>(j & 1 ? c0[j / 2] >> 16 : c0[j / 2] & 0xffffu));
+            const float cj1 = h2f(static_cast<uint16_t>(j & 1 ? c1[j / 2] >> 16 : c1[j / 2] & 0xffffu));
+            const uint32_t v = static_cast<uint32_t>(f2h(x0 * cj0)) | (static_cast<uint32_t>(f2h(x1 * cj1)) << 16);
+            const uint32_t amax = wave_umax(max(v & 0x7fffu, (v >> 16) & 0x7fffu));
+            const int eh = min(max(static_cast<int>(amax >> 10), 1), 30);
+            const int e = 20 - eh;
+            if (blk == j)
+                scale_mine = __uint_as_float(static_cast<uint32_t>(126 - e) << 23);
+            const int va = __builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x50, 0xF, 0xF, true);   // quad_perm 0,0,1,1
+            const int vb = __builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xFA, 0xF, 0xF, true);   // quad_perm 2,2,3,3
+            v2h z = as_v2h(__builtin_amdgcn_perm(static_cast<uint32_t>(vb), static_cast<uint32_t>(va), half_sel));
+            const float sc = __uint_as_float(static_cast<uint32_t>(127 - e - fac_log2) << 23);
+            const float sc_last = __uint_as_float(static_cast<uint32_t>(127 - 8 - e - fac_log2) << 23);
+            v2s b = {0, 0};
+            b = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(b, z, sc, false);
+            z -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(as_int(b), sc, false);
+            b = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(b, z, sc, true);
+            z -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(as_int(b), sc, true);
+            const v2s b3 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(v2s{0, 0}, z, sc_last, false);
+            *reinterpret_cast<short *>(img + off + (j * 4 + 0) * 32) = b[0];
+            *reinterpret_cast<short *>(img + off + (j * 4 + 1) * 32) = b[1];
+            *reinterpret_cast<short *>(img + off + (j * 4 + 2) * 32) = b3[0];
+        }
+        const v8i A = *reinterpret_cast<const v8i *>(img + lane * 32);
+        v8i Aj[S];
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+                Aj[j][q] = row_plane == j ? A[q] : 0;
+
+        // -- the units: per column word, transposed words of the two row halves -> B operands of its two tiles
+#pragma unroll
+        for (int h = 0; h < NWW; ++h) {
+            v4f D[2];
+            D[0] = v4f{0.f, 0.f, 0.f, 0.f};
+            D[1] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < S; ++j) {
+                const uint32_t ta = transpose_16x16_blocks_across_lanes(wa[h][j], lane);
+                const uint32_t tb = transpose_16x16_blocks_across_lanes(wb[h][j], lane);
+                const uint32_t pr[2] = {(ta & 0xffffu) | (tb << 16), (ta >> 16) | (tb & 0xffff0000u)};
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const uint32_t w = pr[t];
+                    v8i B;
+                    B[0] = static_cast<int>(w & 0x11111111u);
+                    B[1] = static_cast<int>(w & 0x22222222u);
+                    B[2] = static_cast<int>(w & 0x44444444u);
+                    B[3] = static_cast<int>((w >> 1) & 0x44444444u);
+                    B[4] = 0; B[5] = 0; B[6] = 0; B[7] = 0;
+                    D[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(Aj[j], B, D[t], 0, 4, 0, 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                acc[h][t] = fmaf(fmaf(D[t][2], 1.f / kLastTermScale, D[t][0] + D[t][1]), scale_mine, acc[h][t]);
+        }
+        if (more)
+            gather_lines(raw_next, n0, n1);
+    }
+#pragma unroll
+    for (int h = 0; h < NWW; ++h)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+            red[wave][h * 2 + t][lane] = acc[h][t];
+    __syncthreads();
+    // tile by tile (the first waves take one each): over the waves, then over the four planes (lane groups)
+    for (int tile = wave; tile < 2 * NWW; tile += waves) {      // wave-uniform
+        float total = 0.f;
+        for (int w = 0; w < waves; ++w)
+            total += red[w][tile][lane];
+        red[0][tile][lane] = total;           // (the first row's slot of this tile: read above, by this lane only)
+        __builtin_amdgcn_s_waitcnt(0xc07f);    // lgkmcnt(0)
+        __builtin_amdgcn_wave_barrier();
+        if (lane < 16) {
+            float sum = (red[0][tile][lane] + red[0][tile][lane + 16]) + (red[0][tile][lane + 32] + red[0][tile][lane + 48]);
+            const int n = (nw0 + (tile >> 1)) * 32 + (tile & 1) * 16 + lane;
+            if (n < N) {
+                const size_t at = static_cast<size_t>(m) * N + n;
+                bool mine_to_store = true;
+                if (ksplit > 1) {
+                    unsigned long long tot = (1ull << 56) + static_cast<unsigned long long>(to_fixed(sum) + kAccBias);
+                    tot += __hip_atomic_fetch_add(acc_words + at, tot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    mine_to_store = static_cast<int>(tot >> 56) == ksplit;
+                    if (mine_to_store) {
+                        const long long fixed = static_cast<long long>(tot & ((1ull << 56) - 1)) - (static_cast<long long>(ksplit) << 47);
+                        const float hi = static_cast<float>(static_cast<int>(fixed >> 24));
+                        const float lo = static_cast<float>(static_cast<int>(fixed & 0xffffff));
+                        sum = fmaf(hi, 1.f / (1 << (kAccFracBits - 24)), lo * (1.f / (1 << kAccFracBits)));
+                        __hip_atomic_store(acc_words + at, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+                if (mine_to_store) {
+                    uint16_t r = f2h(sum);
+                    if (bias)
+                        r = hadd(r, bias[n]);
+                    out[at] = r;
+                }
+            }
+        }
+    }
+}
+
 template <typename LIdxT, typename RIdxT>
 __global__ void __launch_bounds__(256)
 sbvr_mm_T_kernel(const uint32_t *__restrict__ l_bvr, const void *__restrict__ l_idx,
@@ -2780,10 +3003,10 @@ int sbvr_hip_linear_f16_stream_floor(const uint32_t *bvr, const void *coeff_idx,
                        workspace_bytes, 0, stream, Prologue{kXFloor, nullptr, nullptr, nullptr, 0.f});
 }
 
-int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_coeff_idx,
-                          int idx_bytes, const void *r_coeff_cache, const void *bias,
-                          void *out, int M, int N, int K, int S, int G, int L,
-                          void *stream)
+int sbvr_hip_row_deq_mm_T_ws(const void *x, const uint32_t *r_bvr, const void *r_coeff_idx,
+                             int idx_bytes, const void *r_coeff_cache, const void *bias,
+                             void *out, int M, int N, int K, int S, int G, int L,
+                             void *workspace, size_t workspace_bytes, void *stream)
 {
     if (!x || !r_bvr || !r_coeff_idx || !r_coeff_cache || !out)
         return fail(SBVR_HIP_EINVAL, "null pointer argument");
@@ -2796,8 +3019,44 @@ int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_co
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (idx_bytes == 1 && L > 256)
         return fail(SBVR_HIP_EINVAL, "uint8 indices cannot address L=%d lines", L);
-    if (M <= 65535 && (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) && reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0 &&
-        reinterpret_cast<uintptr_t>(r_coeff_cache) % 16 == 0) {
+    const bool tables_aligned = reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0 && reinterpret_cast<uintptr_t>(r_coeff_cache) % 16 == 0;
+    if (M <= 65535 && S == 4 && K % kSub == 0 && G % 64 == 0 && tables_aligned && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&
+        reinterpret_cast<uintptr_t>(r_coeff_idx) % 4 == 0 && !env_switches().rowdeq_lanes) {
+        // plane sums on the matrix cores over bits transposed across lanes
+        const int nsub = K / kSub;
+        // (128 columns per workgroup, one A image for twice the columns, measured slower: 17.3 against 15.6 us at
+        // 4096 -> 14336: it wants more than 128 registers)
+        const int nww = 2;
+        const long col_wgs = static_cast<long>((N / 32 + nww - 1) / nww) * M;
+        // K in as many parts as give the CUs a workgroup each, if the caller brought the accumulators
+        int ksplit = 1;
+        if (workspace && reinterpret_cast<uintptr_t>(workspace) % 8 == 0 &&
+            workspace_bytes >= static_cast<size_t>(M) * N * sizeof(unsigned long long)) {
+            // (measured at 4096 -> 4096 / 14336 -> 4096, 64 column workgroups: 13.2 / 39.0 us unsplit, 7.1 / 14.1 in 4
+            // parts, 7.2 / 18.5 in 8; at 4096 -> 14336, 224 of them: 15.3 unsplit, 18.4 in 2)
+            while (ksplit < 32 && col_wgs * ksplit < 3L * current_cus() / 4 && nsub / (ksplit * 2) >= 4)
+                ksplit *= 2;
+        }
+        const int per_part = (nsub + ksplit - 1) / ksplit;
+        ksplit = (nsub + per_part - 1) / per_part;              // (no empty parts)
+        const int waves = per_part < kRowDeqWaves ? per_part : kRowDeqWaves;
+        const dim3 grid(static_cast<unsigned>((N / 32 + nww - 1) / nww), static_cast<unsigned>(M), static_cast<unsigned>(ksplit)), block(64 * waves);
+        if (nww == 4)
+            hipLaunchKernelGGL(sbvr_row_deq_mfma_kernel<4>, grid, block, 0, st, static_cast<const uint16_t *>(x), r_bvr, r_coeff_idx,
+                               static_cast<const uint16_t *>(r_coeff_cache), static_cast<const uint16_t *>(bias),
+                               static_cast<uint16_t *>(out), static_cast<unsigned long long *>(workspace), M, N, K, L, G,
+                               idx_bytes == 2 ? 1 : 0, ksplit);
+        else
+            hipLaunchKernelGGL(sbvr_row_deq_mfma_kernel<2>, grid, block, 0, st, static_cast<const uint16_t *>(x), r_bvr, r_coeff_idx,
+                               static_cast<const uint16_t *>(r_coeff_cache), static_cast<const uint16_t *>(bias),
+                               static_cast<uint16_t *>(out), static_cast<unsigned long long *>(workspace), M, N, K, L, G,
+                               idx_bytes == 2 ? 1 : 0, ksplit);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return fail(SBVR_HIP_ELAUNCH, "row_deq launch: %s", hipGetErrorString(e));
+        return SBVR_HIP_OK;
+    }
+    if (M <= 65535 && (S == 2 || S == 3 || S == 4 || S == 6 || S == 8) && tables_aligned) {
         // lanes along K; as many waves as there are steps of 64 rows, up to kRowDeqWaves
         const int steps = (K + 63) / 64;
         const int waves = steps < kRowDeqWaves ? steps : kRowDeqWaves;
@@ -2832,6 +3091,19 @@ int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_co
     if (e != hipSuccess)
         return fail(SBVR_HIP_ELAUNCH, "row_deq launch: %s", hipGetErrorString(e));
     return SBVR_HIP_OK;
+}
+
+int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_coeff_idx,
+                          int idx_bytes, const void *r_coeff_cache, const void *bias,
+                          void *out, int M, int N, int K, int S, int G, int L,
+                          void *stream)
+{
+    return sbvr_hip_row_deq_mm_T_ws(x, r_bvr, r_coeff_idx, idx_bytes, r_coeff_cache, bias, out, M, N, K, S, G, L, nullptr, 0, stream);
+}
+
+size_t sbvr_hip_row_deq_mm_T_workspace(int M, int N)
+{
+    return M > 0 && N > 0 ? static_cast<size_t>(M) * N * sizeof(unsigned long long) : 0;
 }
 
 int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_bytes,

@@ -230,9 +230,12 @@ torch::Tensor sbvr_row_deq_mm_T(torch::Tensor l_w, torch::Tensor r_bvr, torch::T
     TORCH_CHECK(G * r_coeff_idx.size(0) == N, "r_coeff_idx has ", r_coeff_idx.size(0), " groups, N=", N);
     const DeviceGuard guard(l_w.device());
     auto out = torch::empty({M, N}, torch::dtype(torch::kFloat16).device(l_w.device()));
-    check(sbvr_hip_row_deq_mm_T(l_w.data_ptr(), static_cast<const uint32_t *>(r_bvr.data_ptr()), r_coeff_idx.data_ptr(), ib,
-                                r_coeff_cache.data_ptr(), bias_ptr(bias, N, l_w), out.data_ptr(), M, N, K, S, G, L,
-                                current_stream()));
+    hipStream_t stream = current_stream();
+    const size_t need = sbvr_hip_row_deq_mm_T_workspace(static_cast<int>(M), static_cast<int>(N));
+    torch::Tensor ws = workspace(need, l_w, stream);
+    check(sbvr_hip_row_deq_mm_T_ws(l_w.data_ptr(), static_cast<const uint32_t *>(r_bvr.data_ptr()), r_coeff_idx.data_ptr(), ib,
+                                   r_coeff_cache.data_ptr(), bias_ptr(bias, N, l_w), out.data_ptr(), M, N, K, S, G, L,
+                                   ws.data_ptr(), need, stream));
     return out;
 }
 

@@ -54,6 +54,9 @@ def _load():
     lib.sbvr_hip_linear_f16_noalloc.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, vp]
     lib.sbvr_hip_linear_f16_stream_floor.argtypes = [vp, vp, i, vp, vp, i, i, i, i, i, vp, sz, vp]
     lib.sbvr_hip_row_deq_mm_T.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp]
+    lib.sbvr_hip_row_deq_mm_T_ws.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
+    lib.sbvr_hip_row_deq_mm_T_workspace.restype = sz
+    lib.sbvr_hip_row_deq_mm_T_workspace.argtypes = [i, i]
     lib.sbvr_hip_mm_T.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
     fp = ctypes.POINTER(ctypes.c_float)
     lib.sbvr_hip_dec_add_rmsnorm_f16.argtypes = [vp, vp, vp, vp, i, ctypes.c_float, vp]
@@ -263,9 +266,11 @@ def _sbvr_row_deq_mm_T(l_w, r_bvr, r_coeff_idx, r_coeff_cache, bias, use_shfl=0,
     ib = _idx_bytes(r_coeff_idx, L, "r_coeff_idx")
     out = torch.empty((M, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
-        _check(lib.sbvr_hip_row_deq_mm_T(l_w.data_ptr(), r_bvr.data_ptr(), r_coeff_idx.data_ptr(), ib,
-                                         r_coeff_cache.data_ptr(), _bias_ptr(bias, N, dev), out.data_ptr(),
-                                         M, N, K, S, G, L, _stream()))
+        need = lib.sbvr_hip_row_deq_mm_T_workspace(M, N)
+        ws = _workspace(need, dev)
+        _check(lib.sbvr_hip_row_deq_mm_T_ws(l_w.data_ptr(), r_bvr.data_ptr(), r_coeff_idx.data_ptr(), ib,
+                                            r_coeff_cache.data_ptr(), _bias_ptr(bias, N, dev), out.data_ptr(),
+                                            M, N, K, S, G, L, ws.data_ptr(), need, _stream()))
     return out
 
 

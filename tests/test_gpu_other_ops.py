@@ -63,7 +63,10 @@ def test_mm_T_object_api(oracle, golden):
 @pytest.mark.parametrize("M,N,K,S,G,L", [(1, 256, 64, 4, 256, 9), (2, 512, 40, 2, 128, 300),
                                          (3, 1024, 4096, 4, 128, 256), (1, 96, 1000, 3, 32, 700),
                                          (5, 64, 130, 8, 64, 40), (1, 4096, 2048, 6, 128, 256),
-                                         (2, 14336, 512, 4, 128, 256), (1, 32, 1, 4, 32, 2)])
+                                         (2, 14336, 512, 4, 128, 256), (1, 32, 1, 4, 32, 2),
+                                         # four planes, K a multiple of 128, groups of 64 columns and more: the MFMA form
+                                         (1, 64, 128, 4, 64, 5), (4, 256, 640, 4, 64, 300), (2, 192, 256, 4, 192, 9),
+                                         (1, 14336, 4096, 4, 128, 256), (1, 4096, 14336, 4, 256, 256)])
 def test_row_deq_mm_T(oracle, M, N, K, S, G, L):
     import sbvr
     dev = torch.device("cuda:0")
@@ -77,6 +80,35 @@ def test_row_deq_mm_T(oracle, M, N, K, S, G, L):
     want = oracle.C.row_deq_mm_T(x, bvr, idx, cache, G, bias).astype(np.float64)
     d = np.abs(y.float().cpu().numpy().astype(np.float64) - want)
     assert d.max() <= 2.0 ** -9 * max(np.abs(want).max(), 1.0)
+
+
+def test_row_deq_mm_T_without_workspace_and_repeatable(oracle):
+    """The reference-shaped entry point (no workspace: K is never split across workgroups) against the oracle at a
+    shape the binding would split, and the split form twice: the fixed-point accumulators make it repeatable."""
+    import ctypes
+    import sbvr
+    from sbvr import hip
+    dev = torch.device("cuda:0")
+    M, N, K, S, G, L = 2, 1024, 2048, 4, 128, 256
+    rng = np.random.default_rng(5)
+    bvr, idx, cache = _rand_enc(rng, K, N, S, G, L, oracle)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    dx, db, di, dc = t(x), t(bvr), t(idx), t(cache)
+    out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    lib = hip._load()
+    vp = ctypes.c_void_p
+    rc = lib.sbvr_hip_row_deq_mm_T(vp(dx.data_ptr()), vp(db.data_ptr()), vp(di.data_ptr()), 1, vp(dc.data_ptr()), None,
+                                   vp(out.data_ptr()), M, N, K, S, G, L, vp(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    want = oracle.C.row_deq_mm_T(x, bvr, idx, cache, G, None).astype(np.float64)
+    assert np.abs(out.float().cpu().numpy() - want).max() <= 2.0 ** -9 * max(np.abs(want).max(), 1.0)
+    none = torch.zeros(0, dtype=torch.float16, device=dev)
+    first = sbvr._sbvr_row_deq_mm_T(dx, db, di, dc, none, 0, bvr_len=G)
+    assert np.abs(first.float().cpu().numpy() - want).max() <= 2.0 ** -9 * max(np.abs(want).max(), 1.0)
+    for _ in range(4):
+        assert torch.equal(first, sbvr._sbvr_row_deq_mm_T(dx, db, di, dc, none, 0, bvr_len=G))
 
 
 def test_row_deq_golden(oracle, golden):
