@@ -1119,8 +1119,10 @@ GemvPlan plan_gemv_uncached(int M, int N, int K, int S, int cus, int min_waves)
     }
     if (best.CT == 0) {
         const long units = static_cast<long>(tiles16) * nsub;
-        int want = units >= 8L * 2048 ? 4 : (units >= 2L * 2048 ? 2 : 1);
-        while (want > 1 && !shape_ok_for(MT, want, 1))
+        // (8 units per wave for the largest matrices: 14336 -> 4096 measured 8.2-8.3 us with 4 tiles x 2 sub-groups
+        // against 8.6-8.7 with 4 x 1)
+        int want = units >= 12L * 2048 && MT == 1 ? 8 : (units >= 8L * 2048 ? 4 : (units >= 2L * 2048 ? 2 : 1));
+        while (want > 1 && want <= 4 && !shape_ok_for(MT, want, 1))
             want /= 2;
         double best_cost = 1e30;
         for (int i = 0; i < kNumShapes; ++i) {
