@@ -1,7 +1,8 @@
 // libsbvr_hip.so -- HIP kernels for gfx950 (MI355X) behind the C ABI of
 // include/sbvr_hip.h: the SBVR compressed-domain linear layer.
 //
-// Decode path (M <= 16), sbvr_gemv_mfma_kernel.  The work is one bit per weight
+// Decode path (M <= 16), sbvr_gemv_mfma_kernel (and, for 5..16 rows, sbvr_gemv_batch_kernel, whose waves share
+// the activation operands of a sub-group).  The work is one bit per weight
 // element and plane, far too many bits for one VALU lane-op each, so the masked
 // sums run on the matrix cores:
 //   * a 32-bit plane word becomes four dwords of fp4 (e2m1) values with one AND
@@ -30,12 +31,13 @@
 // activations into A operands: sbvr_hip_linear_f16_swiglu / _add_rmsnorm.
 //
 // Prefill path (M > 32), sbvr_gemm_mfma_kernel: weights decoded to fp16 tiles
-// in LDS, fp16 MFMA, fp32 accumulation; sbvr_gemm_rows32_kernel for 9..32 rows
+// in LDS, fp16 MFMA, fp32 accumulation; sbvr_gemm_rows32_kernel for 17..32 rows
 // (the batch rows are the 32 rows of one MFMA, weights decoded in registers).
 //
 // The reference's own operator forms: sbvr_mm_T_popc_kernel (both operands
-// encoded: popcounts per group, lane per column) and sbvr_row_deq_lanes_kernel
-// (trans=True weight, lanes along K).
+// encoded: popcounts per group, lane per column), sbvr_row_deq_mfma_kernel (trans=True
+// weight: bits transposed across lanes, then the decode path's plane sums) and
+// sbvr_row_deq_lanes_kernel (the same for other plane counts, lanes along K).
 //
 // Portable kernels (any shape, one thread per output) back all of them.
 #include <hip/hip_runtime.h>
@@ -1969,8 +1971,9 @@ bool rows32_path_ok(int M, int N, int K, int S, int G)
 }
 
 // Measured on MI355X at the Llama-3-8B shapes: the 32-row kernel takes about the same
-// time for any batch up to 32 (24 us at 4096 -> 14336), the decode kernel 17 us at 8 rows
-// and 34 us at 16; with fewer than one 32-column workgroup per CU the 32-row kernel loses.
+// time for any batch up to 32 (24-25 us at 4096 -> 14336), the decode kernels 13 us at 8 rows
+// and 21 us at 16: the 32-row kernel is for 17..32 rows, and for 5..16 rows of shapes the
+// decode kernels do not cover.
 bool rows32_preferred(int M, int N, int K, int S, int G, int cus)
 {
     (void)cus;
