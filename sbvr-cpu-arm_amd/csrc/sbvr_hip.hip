@@ -466,6 +466,11 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
         for (int sgi = 0; sgi < SP; ++sgi)
             xw[sgi] = reinterpret_cast<const uint32_t *>(a.norm_w + static_cast<size_t>(sg0 + sgi) * kSub)[lane];
+        // (the waves meet before any of them asks for plane words: every wave's share of x is then ahead of
+        // all of those in the CU's queue; no fence, nothing has been written yet.  0.1-0.15 us per launch)
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
     }
     // line indices: one load per sub-group and 64 columns of the window, lane l takes the index of column
     // n_base + 64*iw + l; they are handed to the (tile, column) lanes later, in LDS permutes: every
@@ -1060,7 +1065,7 @@ const EnvSwitches &env_switches()
 }
 
 // (CT, SP) pairs that have a kernel instance; see the dispatch below.
-constexpr int kShapes[][2] = {{1, 1}, {1, 2}, {1, 4}, {1, 7}, {2, 1}, {2, 2}, {2, 4}, {2, 7}, {4, 1}, {4, 2}, {4, 4}};
+constexpr int kShapes[][2] = {{1, 1}, {1, 2}, {1, 4}, {1, 7}, {2, 1}, {2, 2}, {2, 4}, {2, 7}, {4, 1}, {4, 2}, {4, 4}, {7, 2}};
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
 
 constexpr bool shape_ok_for(int MT, int CT, int SP)
@@ -1107,8 +1112,11 @@ GemvPlan plan_gemv_uncached(int M, int N, int K, int S, int cus, int min_waves)
     const int wg_waves = norm ? 8 : kMaxWaves;
     if (best.CT == 0 && eCT <= 0 && nsub % wg_waves == 0 && wg_waves >= min_waves && N >= (norm ? 64 : 16) * cus) {
         const int SP = nsub / wg_waves;
-        // windows of wstride columns, r workgroups per CU
-        for (int r = (N + 64 * cus - 1) / (64 * cus); r <= 4; ++r) {
+        // windows of wstride columns, r workgroups per CU; without the prologue one workgroup per CU takes up
+        // to 7 tiles (4096 -> 28672: 256 windows of 112 columns 11.8 us, 512 of 56 columns 13.1-13.5 us; with
+        // the prologue, whose barrier 16 waves feel more than 8, the two measured the same)
+        const int widest = norm ? 64 : 112;
+        for (int r = (N + widest * cus - 1) / (widest * cus); r <= 4; ++r) {
             const int wstride = ((N + cus * r - 1) / (cus * r) + 7) / 8 * 8;
             const int CT = (wstride + 15) / 16;
             if (wstride < 16)
@@ -1231,7 +1239,7 @@ hipError_t launch_gemv_shape(const GemvArgs &a, const GemvPlan &p, hipStream_t s
             return launch_gemv_inst<S, MT, ct, sp, XM>(a, p, st)
     SBVR_SHAPE(1, 1); SBVR_SHAPE(1, 2); SBVR_SHAPE(1, 4); SBVR_SHAPE(1, 7);
     SBVR_SHAPE(2, 1); SBVR_SHAPE(2, 2); SBVR_SHAPE(2, 4); SBVR_SHAPE(2, 7);
-    SBVR_SHAPE(4, 1); SBVR_SHAPE(4, 2); SBVR_SHAPE(4, 4);
+    SBVR_SHAPE(4, 1); SBVR_SHAPE(4, 2); SBVR_SHAPE(4, 4); SBVR_SHAPE(7, 2);
 #undef SBVR_SHAPE
     return hipErrorInvalidConfiguration;
 }
@@ -2269,7 +2277,7 @@ sbvr_row_deq_mfma_kernel(const uint16_t *__restrict__ x, const uint32_t *__restr
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int waves = static_cast<int>(blockDim.x >> 6);
-    const int col = lane & 15, blk = lane >> 4;
+    const int blk = lane >> 4;
     const int m = blockIdx.y;
     const int nwords = N / 32;
     const int nw0 = NWW * blockIdx.x;                     // the workgroup's NWW column words (the last ones may be missing)

@@ -88,6 +88,14 @@ def test_llama_shapes(oracle, N, K):
     run_case(oracle, N, K, 4, 128, 1, 256, seed=11)
 
 
+@pytest.mark.parametrize("N,S,M,L,bias", [(28672, 4, 1, 256, False), (28672, 2, 3, 256, False), (28672, 3, 4, 300, False),
+                                          (27000, 4, 2, 256, False), (26000, 4, 1, 300, True), (28672, 8, 1, 256, False)])
+def test_one_window_per_cu_up_to_seven_tiles(oracle, N, S, M, L, bias):
+    # the fused gate|up width: on 256 CUs one workgroup per CU takes all of K for a window of 104-112 columns
+    # (7 column tiles, the last one partly its neighbour's at 104; at 27000 the last window is moved left)
+    run_case(oracle, N, 4096, S, 128, M, L, seed=N + S + M, bias=bias)
+
+
 @pytest.mark.parametrize("S", [2, 3, 4])
 @pytest.mark.parametrize("M", [2, 16])
 def test_sweep_gate(oracle, S, M):
