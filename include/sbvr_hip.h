@@ -208,6 +208,26 @@ int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_byte
                   const void *bias, void *out, int M, int N, int K, int Sl, int Sr,
                   int G, int Ll, int Lr, void *stream);
 
+/*
+ * The same product with room for a split of K across workgroups: a workspace of
+ * sbvr_hip_mm_T_workspace(M, N) bytes (M*N 64-bit accumulators, zero-filled once, 8-byte aligned,
+ * left zero by every call; it may be the workspace of sbvr_hip_linear_f16, not used by two calls
+ * at once).  One left row of up to 4 planes (the case the reference's kernels are written for,
+ * sbvr_kernel.cu:464-562) at the decode kernel's shapes (N >= 16, K and G multiples of 128, G / 128
+ * a power of two, 2, 3, 4, 6 or 8 right planes) runs on that kernel: the left operand's planes,
+ * each times its coefficient, are its batch rows, the popcounts come out of the matrix cores and the
+ * rows are added up in fp32 before the one rounding.  Where that launch splits K across workgroups
+ * (N = 4096 at K = 14336 on an MI355X) it needs the workspace; without one, and for every other
+ * shape, the popcount kernels of sbvr_hip_mm_T run.  The reference's operator has no such argument
+ * (sbvr_ops.cpp:35-76); its bindings here bring their own.
+ */
+int sbvr_hip_mm_T_ws(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_bytes,
+                     const void *l_coeff_cache, const uint32_t *r_bvr,
+                     const void *r_coeff_idx, int r_idx_bytes, const void *r_coeff_cache,
+                     const void *bias, void *out, int M, int N, int K, int Sl, int Sr,
+                     int G, int Ll, int Lr, void *workspace, size_t workspace_bytes, void *stream);
+size_t sbvr_hip_mm_T_workspace(int M, int N);
+
 #ifdef __cplusplus
 }
 #endif

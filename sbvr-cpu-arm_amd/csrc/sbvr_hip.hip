@@ -34,8 +34,10 @@
 // in LDS, fp16 MFMA, fp32 accumulation; sbvr_gemm_rows32_kernel for 17..32 rows
 // (the batch rows are the 32 rows of one MFMA, weights decoded in registers).
 //
-// The reference's own operator forms: sbvr_mm_T_popc_kernel (both operands
-// encoded: popcounts per group, lane per column), sbvr_row_deq_mfma_kernel (trans=True
+// The reference's own operator forms: both operands encoded: the decode kernel
+// with the left operand's planes as batch rows (one left row of up to 4 planes),
+// else sbvr_mm_T_popc_kernel (popcounts per group, lane per column);
+// sbvr_row_deq_mfma_kernel (trans=True
 // weight: bits transposed across lanes, then the decode path's plane sums) and
 // sbvr_row_deq_lanes_kernel (the same for other plane counts, lanes along K).
 //
@@ -176,6 +178,11 @@ struct GemvArgs {
     const uint16_t *norm_w;     // XM == 2: RMSNorm weight
     uint16_t *x_out;            // XM == 2: receives fp16(x + delta)
     float eps;
+    // XM == kXPlanes: the left operand, SBVR-encoded (one row, M planes, default layout)
+    const uint32_t *xbvr;       // (K / 32, 1, M)
+    const void *xidx;           // (K / G, 1)
+    const uint16_t *xcache;     // (xL, M)
+    int x_idx16, xL;
 #ifdef SBVR_TRACE
     unsigned long long *trace;   // 8 timestamps per workgroup (development builds only)
 #endif
@@ -341,6 +348,11 @@ __device__ __forceinline__ float wave_fsum(float v)
 //             to x_out.
 constexpr int kXPlain = 0, kXSwiGLU = 1, kXAddNorm = 2, kXAddNorm2 = 3;   // (3: two chunks of x per thread for the norm)
 constexpr int kXFloor = 4;      // measurement aid: the launch's plane-word and index requests only, no arithmetic, no output
+// kXPlanes: the left operand is SBVR-encoded as well (one left row of M <= 4 planes, the reference's both-encoded
+//           product, sbvr_kernel.cu:464-562): batch row r of the A operands is plane r times its coefficient, a_r
+//           or 0 per element (exact in fp16, hence in the three fp8 terms), so the MFMAs give
+//           sum_k a_r L_r[k] R_j[k] = a_r * popcount(L_r & R_j) per sub-group, and the rows are added up at the end.
+constexpr int kXPlanes = 5;
 constexpr int kNormChunksMax = 2;             // 16-byte chunks of x a thread sums for the norm, at most
 
 __device__ __forceinline__ uint32_t swiglu_pair(uint32_t g, uint32_t u)
@@ -438,6 +450,27 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     v4u sx[NV], sd[NV];                                                 // this thread's share of all of x and delta
     if constexpr (XM == kXFloor) {
         // (no activations)
+    } else if constexpr (XM == kXPlanes) {
+        // lane l holds elements 2l, 2l + 1 of a sub-group: bits 2 (l % 16) and + 1 of its word l / 16
+#pragma unroll
+        for (int sgi = 0; sgi < SP; ++sgi) {
+            const int sg = sg0 + sgi;
+            const int g = sg >> a.gshift;
+            const int lline = a.x_idx16 ? static_cast<int>(static_cast<const uint16_t *>(a.xidx)[g])
+                                        : static_cast<int>(static_cast<const uint8_t *>(a.xidx)[g]);
+            const uint16_t *la = a.xcache + static_cast<size_t>(min(lline, a.xL - 1)) * a.M;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    xx[sgi][mt][r] = 0u;
+                    if (mt == 0 && r < a.M) {                       // wave-uniform
+                        const uint32_t w = a.xbvr[(static_cast<size_t>(4 * sg) + blk) * a.M + r];
+                        const uint32_t two = (w >> (2 * col)) & 3u;
+                        xx[sgi][mt][r] = __umul24((two & 1u) | ((two & 2u) << 15), static_cast<uint32_t>(la[r]));
+                    }
+                }
+        }
     } else if constexpr (!kNorm) {
 #pragma unroll
         for (int sgi = 0; sgi < SP; ++sgi)
@@ -585,7 +618,7 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     __builtin_amdgcn_s_setprio(3);
     v8i A[SP][MT];
     float scale[SP][MT];         // of this lane's batch row (blk)
-    const int m_rows = XM != kXPlain ? 1 : a.M;
+    const int m_rows = XM == kXPlain || XM == kXPlanes ? a.M : 1;
     // Lane l = 4g + t of a row's 64 takes elements 8g + t and 8g + t + 4 of the sub-group: the same bit t of two
     // neighbouring nibbles of a plane word, which are neighbouring bytes of the A image (one 16-bit store per
     // term) and share the weight of their B digits (0.5, 1, 2, 2 for t = 0..3, made up for here: 4, 2, 1, 1).
@@ -752,8 +785,12 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
         float total = 0.f;
         for (int w = 0; w < waves; ++w)
             total += red[w * kRedStride + o * 64 + lane];
+        if constexpr (XM == kXPlanes) {      // the rows are the left operand's planes: the output is their sum
+            total += __shfl_xor(total, 16, 64);
+            total += __shfl_xor(total, 32, 64);
+        }
         const int n = n_base + ct * 16 + col, m = mt * 4 + blk;
-        const bool valid = m < a.M && (!shifted || n >= n_own) && n < n_own + a.wstride;
+        const bool valid = (XM == kXPlanes ? m == 0 : m < a.M) && (!shifted || n >= n_own) && n < n_own + a.wstride;
         const size_t at = static_cast<size_t>(m) * N + n;
         if (a.ksplit > 1) {
             // through the accumulators: the adder that completes the count converts
@@ -1256,6 +1293,8 @@ hipError_t launch_gemv_mt(const GemvArgs &a, const GemvPlan &p, int xm, hipStrea
         return p.MT == 1 ? launch_gemv_shape<S, 1, kXAddNorm2>(a, p, st) : hipErrorInvalidConfiguration;
     if (xm == kXFloor)
         return p.MT == 1 ? launch_gemv_shape<S, 1, kXFloor>(a, p, st) : hipErrorInvalidConfiguration;
+    if (xm == kXPlanes)
+        return p.MT == 1 ? launch_gemv_shape<S, 1, kXPlanes>(a, p, st) : hipErrorInvalidConfiguration;
     switch (p.MT) {
     case 1: return launch_gemv_shape<S, 1, kXPlain>(a, p, st);
     case 2: return launch_gemv_shape<S, 2, kXPlain>(a, p, st);
@@ -3119,11 +3158,26 @@ size_t sbvr_hip_row_deq_mm_T_workspace(int M, int N)
     return M > 0 && N > 0 ? static_cast<size_t>(M) * N * sizeof(unsigned long long) : 0;
 }
 
+size_t sbvr_hip_mm_T_workspace(int M, int N)
+{
+    return M > 0 && N > 0 ? static_cast<size_t>(M) * N * sizeof(unsigned long long) : 0;
+}
+
 int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_bytes,
                   const void *l_coeff_cache, const uint32_t *r_bvr,
                   const void *r_coeff_idx, int r_idx_bytes, const void *r_coeff_cache,
                   const void *bias, void *out, int M, int N, int K, int Sl, int Sr,
                   int G, int Ll, int Lr, void *stream)
+{
+    return sbvr_hip_mm_T_ws(l_bvr, l_coeff_idx, l_idx_bytes, l_coeff_cache, r_bvr, r_coeff_idx, r_idx_bytes, r_coeff_cache,
+                            bias, out, M, N, K, Sl, Sr, G, Ll, Lr, nullptr, 0, stream);
+}
+
+int sbvr_hip_mm_T_ws(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_bytes,
+                     const void *l_coeff_cache, const uint32_t *r_bvr,
+                     const void *r_coeff_idx, int r_idx_bytes, const void *r_coeff_cache,
+                     const void *bias, void *out, int M, int N, int K, int Sl, int Sr,
+                     int G, int Ll, int Lr, void *workspace, size_t workspace_bytes, void *stream)
 {
     if (!l_bvr || !l_coeff_idx || !l_coeff_cache || !r_bvr || !r_coeff_idx || !r_coeff_cache || !out)
         return fail(SBVR_HIP_EINVAL, "null pointer argument");
@@ -3139,7 +3193,47 @@ int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_byte
     const uint16_t *lc = static_cast<const uint16_t *>(l_coeff_cache), *rc = static_cast<const uint16_t *>(r_coeff_cache);
     const uint16_t *b = static_cast<const uint16_t *>(bias);
     uint16_t *o = static_cast<uint16_t *>(out);
-    // few left rows (the reference's kernels are written for one): lane-per-column popcount kernel
+    // One left row of up to four planes (what the reference's kernels are written for), at the decode kernel's
+    // shapes: the decode kernel with the left operand's planes as its batch rows; the popcounts come out of the
+    // matrix cores.  4096 -> 14336, 4 x 4 planes: about 9 us against 11.5 us for the popcount kernel below.
+    if (M == 1 && Sl <= 4 && !env_switches().popc_q && mfma_path_ok(Sl, N, K, Sr, G) &&
+        (l_idx_bytes == 2 || Ll <= 256) && (r_idx_bytes == 2 || Lr <= 256) &&
+        reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0 && reinterpret_cast<uintptr_t>(r_coeff_cache) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(l_bvr) % 4 == 0 && reinterpret_cast<uintptr_t>(l_coeff_cache) % 2 == 0) {
+        const GemvPlan p = plan_gemv(Sl, N, K, Sr, current_cus());
+        const size_t need = static_cast<size_t>(N) * sizeof(unsigned long long);
+        const bool room = p.ksplit <= 1 || (workspace && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 8 == 0);
+        if (p.CT > 0 && p.MT == 1 && room) {
+            GemvArgs a{};
+            a.bvr = r_bvr;
+            a.idx = r_coeff_idx;
+            a.cache = rc;
+            a.bias = b;
+            a.out = o;
+            a.M = Sl; a.N = N; a.K = K; a.L = Lr;
+            a.gshift = __builtin_ctz(static_cast<unsigned>(G / kSub));
+            a.idx16 = r_idx_bytes == 2;
+            a.ksplit = p.ksplit;
+            a.xstride = K;
+            a.wstride = p.wstride;
+            a.xbvr = l_bvr;
+            a.xidx = l_coeff_idx;
+            a.xcache = lc;
+            a.x_idx16 = l_idx_bytes == 2;
+            a.xL = Ll;
+            a.acc = p.ksplit > 1 ? static_cast<unsigned long long *>(workspace) : nullptr;
+#ifdef SBVR_TRACE
+            a.trace = g_trace;
+#endif
+            const hipError_t e = launch_gemv(Sr, a, p, kXPlanes, st);
+            if (e != hipSuccess)
+                return fail(SBVR_HIP_ELAUNCH, "mm_T launch through the decode kernel (CT=%d SP=%d waves=%d ksplit=%d): %s", p.CT, p.SP, p.waves,
+                            p.ksplit, hipGetErrorString(e));
+            g_last_kernel = SBVR_HIP_KERNEL_DECODE;
+            return SBVR_HIP_OK;
+        }
+    }
+    // few left rows: lane-per-column popcount kernel
     const int wpg = G / 32;
     if (M <= 64 && (wpg == 1 || wpg == 2 || wpg == 4 || wpg == 8) && Sl >= 2 && Sl <= 4 &&
         reinterpret_cast<uintptr_t>(r_bvr) % 16 == 0 && static_cast<double>(K / 32) * N * Sr < 2147483648.0) {

@@ -207,10 +207,13 @@ torch::Tensor sbvr_mm_T(torch::Tensor l_bvr, torch::Tensor l_coeff_idx, torch::T
     TORCH_CHECK(G * l_coeff_idx.size(0) == K, "coeff_idx has ", l_coeff_idx.size(0), " groups, K=", K);
     const DeviceGuard guard(l_bvr.device());
     auto out = torch::empty({M, N}, torch::dtype(torch::kFloat16).device(l_bvr.device()));
-    check(sbvr_hip_mm_T(static_cast<const uint32_t *>(l_bvr.data_ptr()), l_coeff_idx.data_ptr(), lib,
-                        l_coeff_cache.data_ptr(), static_cast<const uint32_t *>(r_bvr.data_ptr()), r_coeff_idx.data_ptr(),
-                        rib, r_coeff_cache.data_ptr(), bias_ptr(bias, N, l_bvr), out.data_ptr(), M, N, K, Sl, Sr, G, Ll,
-                        Lr, current_stream()));
+    hipStream_t stream = current_stream();
+    const size_t need = sbvr_hip_mm_T_workspace(static_cast<int>(M), static_cast<int>(N));
+    torch::Tensor ws = workspace(need, l_bvr, stream);
+    check(sbvr_hip_mm_T_ws(static_cast<const uint32_t *>(l_bvr.data_ptr()), l_coeff_idx.data_ptr(), lib,
+                           l_coeff_cache.data_ptr(), static_cast<const uint32_t *>(r_bvr.data_ptr()), r_coeff_idx.data_ptr(),
+                           rib, r_coeff_cache.data_ptr(), bias_ptr(bias, N, l_bvr), out.data_ptr(), M, N, K, Sl, Sr, G, Ll,
+                           Lr, ws.data_ptr(), need, stream));
     return out;
 }
 

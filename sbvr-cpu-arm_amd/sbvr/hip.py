@@ -58,6 +58,9 @@ def _load():
     lib.sbvr_hip_row_deq_mm_T_workspace.restype = sz
     lib.sbvr_hip_row_deq_mm_T_workspace.argtypes = [i, i]
     lib.sbvr_hip_mm_T.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
+    lib.sbvr_hip_mm_T_ws.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp, sz, vp]
+    lib.sbvr_hip_mm_T_workspace.restype = sz
+    lib.sbvr_hip_mm_T_workspace.argtypes = [i, i]
     fp = ctypes.POINTER(ctypes.c_float)
     lib.sbvr_hip_dec_add_rmsnorm_f16.argtypes = [vp, vp, vp, vp, i, ctypes.c_float, vp]
     lib.sbvr_hip_dec_attention_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
@@ -296,10 +299,13 @@ def _sbvr_mm_T(l_bvr, l_coeff_idx, l_coeff_cache, r_bvr, r_coeff_idx, r_coeff_ca
     Ll, Lr = l_coeff_cache.shape[0], r_coeff_cache.shape[0]
     out = torch.empty((M, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
-        _check(lib.sbvr_hip_mm_T(l_bvr.data_ptr(), l_coeff_idx.data_ptr(), _idx_bytes(l_coeff_idx, Ll, "l_coeff_idx"),
-                                 l_coeff_cache.data_ptr(), r_bvr.data_ptr(), r_coeff_idx.data_ptr(),
-                                 _idx_bytes(r_coeff_idx, Lr, "r_coeff_idx"), r_coeff_cache.data_ptr(),
-                                 _bias_ptr(bias, N, dev), out.data_ptr(), M, N, K, Sl, Sr, G, Ll, Lr, _stream()))
+        need = lib.sbvr_hip_mm_T_workspace(M, N)
+        ws = _workspace(need, dev)
+        _check(lib.sbvr_hip_mm_T_ws(l_bvr.data_ptr(), l_coeff_idx.data_ptr(), _idx_bytes(l_coeff_idx, Ll, "l_coeff_idx"),
+                                    l_coeff_cache.data_ptr(), r_bvr.data_ptr(), r_coeff_idx.data_ptr(),
+                                    _idx_bytes(r_coeff_idx, Lr, "r_coeff_idx"), r_coeff_cache.data_ptr(),
+                                    _bias_ptr(bias, N, dev), out.data_ptr(), M, N, K, Sl, Sr, G, Ll, Lr,
+                                    ws.data_ptr(), need, _stream()))
     return out
 
 

@@ -27,7 +27,14 @@ def _close(y, yd, ulps=2.0):
                                                  (1, 1000, 160, 4, 4, 32, 16, 256),     # 5 words: a partial chunk
                                                  (1, 130, 4096, 4, 2, 64, 16, 300),     # 16 chunks, uint16 right index
                                                  (2, 200, 14336, 3, 4, 128, 16, 256),   # 7 chunks per wave
-                                                 (1, 96, 512, 4, 4, 512, 8, 8)])        # group longer than a chunk: portable
+                                                 (1, 96, 512, 4, 4, 512, 8, 8),         # group longer than a chunk
+                                                 # one left row of up to 4 planes at the decode kernel's shapes: the
+                                                 # left planes are that kernel's batch rows
+                                                 (1, 256, 1024, 4, 4, 128, 16, 256), (1, 1030, 2048, 3, 4, 128, 300, 300),
+                                                 (1, 48, 512, 2, 3, 256, 7, 9), (1, 4096, 4096, 4, 4, 128, 16, 256),
+                                                 (1, 14336, 4096, 4, 4, 128, 16, 256), (1, 1000, 1024, 1, 8, 128, 5, 40),
+                                                 (1, 4096, 14336, 4, 4, 128, 16, 256),  # K split across workgroups
+                                                 (1, 2048, 7168, 4, 2, 256, 16, 300), (1, 512, 4096, 4, 6, 128, 9, 256)])
 def test_mm_T(oracle, M, N, K, Sl, Sr, G, Ll, Lr):
     import sbvr
     dev = torch.device("cuda:0")
@@ -44,6 +51,37 @@ def test_mm_T(oracle, M, N, K, Sl, Sr, G, Ll, Lr):
     want, _ = oracle.C.mm_T(lb, li, lc, rb, ri, rc, G, bias)
     d = np.abs(yb.float().cpu().numpy().astype(np.float64) - want.astype(np.float64))
     assert d.max() <= 2.0 ** -9 * max(np.abs(want.astype(np.float64)).max(), 1.0)
+
+
+def test_mm_T_without_workspace_and_repeatable(oracle):
+    """The reference-shaped entry point (no workspace) at a shape whose decode launch would split K across
+    workgroups: it must still answer (through the popcount kernel); and the split form twice, bit for bit."""
+    import ctypes
+    import sbvr
+    from sbvr import hip
+    dev = torch.device("cuda:0")
+    M, N, K, S, G, L = 1, 4096, 14336, 4, 128, 256
+    rng = np.random.default_rng(11)
+    lb, li, lc = _rand_enc(rng, M, K, S, G, 16, oracle)
+    rb, ri, rc_ = _rand_enc(rng, N, K, S, G, L, oracle)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    d = [t(a) for a in (lb, li, lc, rb, ri, rc_)]
+    out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    lib = hip._load()
+    vp = ctypes.c_void_p
+    rc = lib.sbvr_hip_mm_T(vp(d[0].data_ptr()), vp(d[1].data_ptr()), 1, vp(d[2].data_ptr()), vp(d[3].data_ptr()),
+                           vp(d[4].data_ptr()), 1, vp(d[5].data_ptr()), None, vp(out.data_ptr()), M, N, K, S, S, G, 16, L,
+                           vp(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    _, yd = oracle.C.mm_T(lb, li, lc, rb, ri, rc_, G)
+    _close(out, yd)
+    none = torch.zeros(0, dtype=torch.float16, device=dev)
+    first = sbvr._sbvr_mm_T(*d, none, bvr_len=G)
+    _close(first, yd)
+    for _ in range(4):
+        again = sbvr._sbvr_mm_T(*d, none, bvr_len=G)
+        assert torch.equal(first, again)
 
 
 def test_mm_T_object_api(oracle, golden):
