@@ -263,6 +263,10 @@ def sweep_leg():
             for m in (1, 2, 4, 8, 16):
                 if not (s == 4 and m == 1):
                     one(n, k, s, m, tag)
+    # beyond the reference's plan: 17 and 32 rows, the range of the 32-row kernel
+    for tag, n, k in (("q/o", 4096, 4096), ("gate", 14336, 4096), ("down", 4096, 14336)):
+        for m in (17, 32):
+            one(n, k, 4, m, tag)
     return rows
 
 

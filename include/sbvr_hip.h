@@ -83,7 +83,12 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  *                   activation operands, where N >= 32 for up to 8 rows, 64 beyond);
  *   32-row kernel   5 <= M <= 32, K and G multiples of 32, same S: taken for
  *                   17..32 rows, and for 5..16 rows of shapes the decode kernel
- *                   does not cover (N < 16, K or G not a multiple of 128);
+ *                   does not cover (N < 16, K or G not a multiple of 128).  For
+ *                   17..32 rows with 2, 3 or 4 planes and K and G multiples of 64
+ *                   it decodes by table look-up (the subset sums of a group's
+ *                   coefficient line) and, with a workspace and few columns,
+ *                   splits K across workgroups through the decode kernel's
+ *                   accumulators; same results as its arithmetic form;
  *   prefill kernel  M > 32 (or 17..32 with flags bit 1), K and G multiples of 64,
  *                   same S; with a workspace and few output tiles, K is split
  *                   across workgroups;

@@ -32,7 +32,8 @@
 //
 // Prefill path (M > 32), sbvr_gemm_mfma_kernel: weights decoded to fp16 tiles
 // in LDS, fp16 MFMA, fp32 accumulation; sbvr_gemm_rows32_kernel for 17..32 rows
-// (the batch rows are the 32 rows of one MFMA, weights decoded in registers).
+// (the batch rows are the 32 rows of one MFMA, weights decoded in registers;
+// sbvr_gemm_rows32_lut_kernel decodes them by table look-up for 2..4 planes).
 //
 // The reference's own operator forms: both operands encoded: the decode kernel
 // with the left operand's planes as batch rows (one left row of up to 4 planes),
@@ -1085,7 +1086,7 @@ struct GemvPlan {
 
 // Development switches, read from the environment once per process.
 struct EnvSwitches {
-    int ct, sp, waves, wstride, show_plan, popc_q, rowdeq_lanes;
+    int ct, sp, waves, wstride, show_plan, popc_q, rowdeq_lanes, lut_rows;
 };
 
 const EnvSwitches &env_switches()
@@ -1096,7 +1097,7 @@ const EnvSwitches &env_switches()
             return v && *v ? atoi(v) : 0;
         };
         return EnvSwitches{get("SBVR_HIP_CT"), get("SBVR_HIP_SP"), get("SBVR_HIP_WAVES"), get("SBVR_HIP_WSTRIDE"),
-                           get("SBVR_HIP_SHOW_PLAN"), get("SBVR_HIP_POPC_Q"), get("SBVR_HIP_ROWDEQ_LANES")};
+                           get("SBVR_HIP_SHOW_PLAN"), get("SBVR_HIP_POPC_Q"), get("SBVR_HIP_ROWDEQ_LANES"), get("SBVR_HIP_LUT_ROWS")};
     }();
     return e;
 }
@@ -1875,6 +1876,10 @@ struct RowsArgs {
     int words_per_group;   // G / 32
     int words_per_wave;    // a multiple of kRowsBlock
     int idx16;
+    // the table look-up form only
+    unsigned long long *acc;   // (M, N) split-K accumulators as in the decode kernel (ksplit > 1)
+    int ksplit;                // workgroups along K (blockIdx.y)
+    int pairs_per_wg;          // word pairs (64 elements of K) of a workgroup
 };
 
 template <int S>
@@ -2044,6 +2049,246 @@ hipError_t launch_rows32(int S, RowsArgs a, hipStream_t st)
     case 3: hipLaunchKernelGGL(sbvr_gemm_rows32_kernel<3>, grid, block, 0, st, a); break;
     case 6: hipLaunchKernelGGL(sbvr_gemm_rows32_kernel<6>, grid, block, 0, st, a); break;
     case 8: hipLaunchKernelGGL(sbvr_gemm_rows32_kernel<8>, grid, block, 0, st, a); break;
+#endif
+    default: return hipErrorInvalidConfiguration;
+    }
+    return hipGetLastError();
+}
+
+// ------------------------------------- MFMA, up to 32 batch rows, weights decoded by table look-up
+//
+// The same contraction as sbvr_gemm_rows32_kernel (batch rows = the 32 rows of v_mfma_f32_32x32x16_f16, 32
+// columns of decoded fp16 weights as B), with a cheaper decode for 2, 3 and 4 planes.  A weight of a group is
+// one of the 2^S subset sums of the group's coefficient line; the lane builds those once per group
+// (sequential fp16 additions in plane order, the sums the arithmetic decode produces bit for bit) and keeps
+// them as byte tables: the low bytes of entries 0..3, 4..7, ... and the high bytes likewise.  A lane owns a
+// whole word of K per step (half h of the wave takes word 2i + h of the word pair i).  Its plane words are
+// merged into four "nibble words" Q_p, p = 0..3: nibble n of Q_p is the S-bit selector of element p + 4n, at
+// the cost of a rotate and an and-or per plane and p.  Then (Q_p >> 0 or 4) & 0x07070707 is four selectors in
+// four bytes, for elements p (+ 4), + 8, + 16, + 24, i.e. a ready v_perm_b32 selector into the byte tables:
+// two permutes fetch the low and the high bytes of four weights (four permutes and two bit-field inserts
+// with 16 entries, where selector bit 3 chooses between the table halves), two more interleave them into
+// packed fp16 pairs.  About 4 VALU operations per weight against 7.5 for the arithmetic decode.
+// The k order inside an MFMA follows from that: elements 2q, 2q+8, 2q+16, 2q+24, 2q+1, 2q+9, 2q+17, 2q+25 of
+// the lane's word for MFMA q = 0..3 of a step; the activations (the lane's batch row, the same 32 elements:
+// 64 bytes, four loads) are put into that order with four permutes per MFMA.
+// K can be split across workgroups (blockIdx.y) through the decode kernel's 64-bit accumulators.
+constexpr int kLutWaves = 8;
+constexpr int kLutMinRows = 17;      // batch rows from which the linear takes this kernel
+
+template <int S>
+__global__ void __launch_bounds__(64 * kLutWaves)
+sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
+{
+    static_assert(S >= 2 && S <= 4, "tables of 4, 8 or 16 entries");
+    __shared__ float red[kLutWaves][16][64];
+    constexpr int CW = (S + 1) / 2;
+    constexpr int TW = S == 4 ? 4 : (S == 3 ? 2 : 1);       // dwords of a byte table
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int N = a.N, K = a.K, M = a.M;
+    const int j = lane & 31, h = lane >> 5;
+    const int n = blockIdx.x * 32 + j, n_ld = min(n, N - 1);
+    const int pairs = K / 64;
+    const int wg_begin = blockIdx.y * a.pairs_per_wg, wg_end = min(pairs, wg_begin + a.pairs_per_wg);
+    const int ppw = (wg_end - wg_begin + kLutWaves - 1) / kLutWaves;
+    const int p_begin = wg_begin + wave * ppw, p_end = min(wg_end, p_begin + ppw);
+    const uint16_t *xrow = a.x + static_cast<size_t>(min(j, M - 1)) * K + 32 * h;      // (rows past M repeat the last one; dropped at the end)
+
+    struct Step {
+        uint32_t w[S];
+        v4u x[4];
+        uint32_t c[CW];
+    };
+    // (loads are never conditional: a pair past the range repeats the last one of K and is not computed)
+    auto load_line = [&](int ip) __attribute__((always_inline)) -> int {
+        const int word = 2 * min(ip, pairs - 1);
+        const size_t at = (static_cast<size_t>(word / a.words_per_group) * N + n_ld) << a.idx16;
+        const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
+        const int lo = ib[at], hi = ib[at + a.idx16];          // two byte loads whatever the width: no branch
+        return lo | (hi << 16);
+    };
+    auto load_step = [&](int ip, Step &st, int line) __attribute__((always_inline)) {
+        const int word = 2 * min(ip, pairs - 1) + h;
+        const Planes<S> pl = load_planes<S, true>(a.bvr + (static_cast<size_t>(word) * N + n_ld) * S);
+#pragma unroll
+        for (int q = 0; q < S; ++q)
+            st.w[q] = pl.w[q];
+        const v4u *xp = reinterpret_cast<const v4u *>(xrow + 64 * min(ip, pairs - 1));
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            st.x[i] = xp[i];
+        const int ln = min(a.idx16 ? (line & 0xff) | ((line >> 8) & 0xff00) : line & 0xff, a.L - 1);
+        load_line_coeffs<S>(a.cache + static_cast<size_t>(ln) * S, st.c);
+    };
+
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        acc[r] = 0.f;
+
+    auto rotr = [](uint32_t v, int r) __attribute__((always_inline)) -> uint32_t {
+        return (r & 31) == 0 ? v : __builtin_amdgcn_alignbit(v, v, r & 31);
+    };
+    auto compute = [&](const Step &st) __attribute__((always_inline)) {
+        // ---- the group's subset sums, entries (2i, 2i + 1) as packed pairs, then as byte tables
+        v2h cc[S];
+#pragma unroll
+        for (int q = 0; q < S; ++q) {
+            const uint32_t bits = q & 1 ? st.c[q / 2] >> 16 : st.c[q / 2] & 0xffffu;
+            cc[q] = as_v2h(bits | (bits << 16));
+        }
+        v2h e[1 << (S - 1)];
+        e[0] = as_v2h((st.c[0] & 0xffffu) << 16);             // entries 0, 1: nothing, c0
+        e[1] = e[0] + cc[1];                                   // 2, 3
+        if constexpr (S >= 3) {
+            e[2] = e[0] + cc[2];                               // 4, 5
+            e[3] = e[1] + cc[2];                               // 6, 7
+        }
+        if constexpr (S == 4) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                e[4 + i] = e[i] + cc[3];                       // 8..15: the last plane is added last
+        }
+        uint32_t tlo[TW], thi[TW];
+#pragma unroll
+        for (int i = 0; i < TW; ++i) {
+            const uint32_t e0 = __builtin_bit_cast(uint32_t, e[2 * i]), e1 = __builtin_bit_cast(uint32_t, e[2 * i + 1]);
+            tlo[i] = __builtin_amdgcn_perm(e1, e0, 0x06040200u);
+            thi[i] = __builtin_amdgcn_perm(e1, e0, 0x07050301u);
+        }
+        // ---- nibble words: nibble n of Q[p] = selector of element p + 4n
+        uint32_t Q[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            uint32_t v = rotr(st.w[0], p) & 0x11111111u;
+            v = (rotr(st.w[1], p - 1) & 0x22222222u) | v;
+            if constexpr (S >= 3)
+                v = (rotr(st.w[2], p - 2) & 0x44444444u) | v;
+            if constexpr (S == 4)
+                v = (rotr(st.w[3], p - 3) & 0x88888888u) | v;
+            Q[p] = v;
+        }
+        // the weights of elements p, p + 8 (first result) and p + 16, p + 24 (second) as packed fp16 pairs
+        auto look_up = [&](int p, uint32_t &w01, uint32_t &w23) __attribute__((always_inline)) {
+            const uint32_t qs = p < 4 ? Q[p & 3] : Q[p & 3] >> 4;
+            const uint32_t sel = qs & (S == 2 ? 0x03030303u : 0x07070707u);
+            uint32_t lo, hi;
+            if constexpr (S == 2) {
+                lo = __builtin_amdgcn_perm(tlo[0], tlo[0], sel);
+                hi = __builtin_amdgcn_perm(thi[0], thi[0], sel);
+            } else {
+                lo = __builtin_amdgcn_perm(tlo[1], tlo[0], sel);
+                hi = __builtin_amdgcn_perm(thi[1], thi[0], sel);
+            }
+            if constexpr (S == 4) {
+                // bytes of ones where selector bit 3 is set: a look-up in the two-entry table {0x00, 0xff}
+                const uint32_t upper = __builtin_amdgcn_perm(0x0000ff00u, 0x0000ff00u, (qs >> 3) & 0x01010101u);
+                const uint32_t lo_u = __builtin_amdgcn_perm(tlo[3], tlo[2], sel), hi_u = __builtin_amdgcn_perm(thi[3], thi[2], sel);
+                lo = (lo_u & upper) | (lo & ~upper);
+                hi = (hi_u & upper) | (hi & ~upper);
+            }
+            w01 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
+            w23 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
+        };
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t b0, b1, b2, b3;
+            look_up(2 * q, b0, b1);
+            look_up(2 * q + 1, b2, b3);
+            const v4u bw = {b0, b1, b2, b3};
+            v4u aw;
+            // dword i of the lane's 64 bytes of activations holds elements 2i, 2i + 1
+            const uint32_t d0 = st.x[0][q], d1 = st.x[1][q], d2 = st.x[2][q], d3 = st.x[3][q];
+            aw.x = __builtin_amdgcn_perm(d1, d0, 0x05040100u);
+            aw.y = __builtin_amdgcn_perm(d3, d2, 0x05040100u);
+            aw.z = __builtin_amdgcn_perm(d1, d0, 0x07060302u);
+            aw.w = __builtin_amdgcn_perm(d3, d2, 0x07060302u);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, aw), __builtin_bit_cast(v8h, bw), acc, 0, 0, 0);
+        }
+    };
+
+    // (two register sets: with three, the loads two steps ahead, the kernel needs 115 registers and was 8-25 % slower)
+    Step s0, s1;
+    int line = load_line(p_begin);
+    load_step(p_begin, s0, line);
+    line = load_line(p_begin + 1);
+    for (int ip = p_begin; ip < p_end; ip += 2) {
+        load_step(ip + 1, s1, line);
+        line = load_line(ip + 2);
+        compute(s0);
+        load_step(ip + 2, s0, line);
+        line = load_line(ip + 3);
+        if (ip + 1 < p_end)
+            compute(s1);
+    }
+
+    // ---- partial results meet in LDS; D[i][jj] sits in lane jj + 32*((i/4)%2), register (i%4) + 4*(i/8)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        red[wave][r][lane] = acc[r];
+    __syncthreads();
+    const uint16_t bias = a.bias && n < N ? a.bias[n] : 0;
+#pragma unroll
+    for (int rr = 0; rr < 16 / kLutWaves; ++rr) {
+        const int r = wave * (16 / kLutWaves) + rr;
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < kLutWaves; ++w)
+            total += red[w][r][lane];
+        const int m = 8 * (r >> 2) + 4 * h + (r & 3);
+        const bool valid = m < M && n < N;
+        const size_t at = static_cast<size_t>(m) * N + n;
+        if (a.ksplit > 1) {
+            unsigned long long tot = (1ull << 56) + static_cast<unsigned long long>(to_fixed(total) + kAccBias);
+            unsigned long long old = 0ull;
+            if (valid)
+                old = __hip_atomic_fetch_add(a.acc + at, tot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            tot += old;
+            if (!valid || static_cast<int>(tot >> 56) != a.ksplit)
+                continue;
+            const long long sum = static_cast<long long>(tot & ((1ull << 56) - 1)) - (static_cast<long long>(a.ksplit) << 47);
+            const float hi = static_cast<float>(static_cast<int>(sum >> 24));
+            const float lo = static_cast<float>(static_cast<int>(sum & 0xffffff));
+            total = fmaf(hi, 1.f / (1 << (kAccFracBits - 24)), lo * (1.f / (1 << kAccFracBits)));
+            __hip_atomic_store(a.acc + at, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (!valid) {
+            continue;
+        }
+        uint16_t v = f2h(total);
+        if (a.bias)
+            v = hadd(v, bias);
+        a.out[at] = v;
+    }
+}
+
+bool lut_path_ok(int M, int N, int K, int S, int G)
+{
+    return M >= 1 && M <= kRowsMax && K % 64 == 0 && G % 64 == 0 && (S == 2 || S == 3 || S == 4) &&
+           static_cast<double>(K / 32) * N * S < 2147483648.0;
+}
+
+// Workgroups along K: until the 32-column blocks times the parts fill the CUs, a wave keeping 4 word pairs and more.
+int lut_ksplit(int N, int K, int cus)
+{
+    const int blocks = (N + 31) / 32, pairs = K / 64;
+    int ks = 1;
+    while (blocks * ks < cus && pairs / (ks * 2) >= 4 * kLutWaves && ks < 16)
+        ks *= 2;
+    return ks;
+}
+
+hipError_t launch_rows32_lut(int S, RowsArgs a, hipStream_t st)
+{
+    const int pairs = a.K / 64;
+    a.pairs_per_wg = (pairs + a.ksplit - 1) / a.ksplit;
+    const dim3 grid(static_cast<unsigned>((a.N + 31) / 32), static_cast<unsigned>(a.ksplit)), block(64 * kLutWaves);
+    switch (S) {
+    case 4: hipLaunchKernelGGL(sbvr_gemm_rows32_lut_kernel<4>, grid, block, 0, st, a); break;
+#ifndef SBVR_FAST_BUILD
+    case 2: hipLaunchKernelGGL(sbvr_gemm_rows32_lut_kernel<2>, grid, block, 0, st, a); break;
+    case 3: hipLaunchKernelGGL(sbvr_gemm_rows32_lut_kernel<3>, grid, block, 0, st, a); break;
 #endif
     default: return hipErrorInvalidConfiguration;
     }
@@ -2778,7 +3023,7 @@ int sbvr_hip_init(int device)
 
 size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G)
 {
-    if (mfma_path_ok(M, N, K, S, G))
+    if (mfma_path_ok(M, N, K, S, G) || lut_path_ok(M, N, K, S, G))
         return static_cast<size_t>(M) * N * sizeof(unsigned long long);
     if (gemm_path_ok(M, N, K, S, G) && !rows32_path_ok(M, N, K, S, G))
         return gemm_workspace_bytes(M, N, K);
@@ -2832,6 +3077,35 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
             if (pro.x_out == x || pro.x_out == pro.delta)
                 return fail(SBVR_HIP_EINVAL, "x_out must not alias x or delta (other workgroups still read them)");
         }
+    }
+    // from kLutMinRows batch rows on, with 2 to 4 planes: the 32-row kernel that decodes by table look-up
+    // (SBVR_HIP_LUT_ROWS moves the threshold: a development switch)
+    const int lut_rows = env_switches().lut_rows > 0 ? env_switches().lut_rows : kLutMinRows;
+    if (pro.mode == kXPlain && !(flags & 3) && aligned && M >= lut_rows && lut_path_ok(M, N, K, S, G) &&
+        reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        RowsArgs r{};
+        r.x = static_cast<const uint16_t *>(x);
+        r.bvr = bvr;
+        r.idx = coeff_idx;
+        r.cache = static_cast<const uint16_t *>(coeff_cache);
+        r.bias = static_cast<const uint16_t *>(bias);
+        r.out = static_cast<uint16_t *>(out);
+        r.M = M; r.N = N; r.K = K; r.L = L;
+        r.words_per_group = G / 32;
+        r.idx16 = idx_bytes == 2;
+        r.ksplit = lut_ksplit(N, K, current_cus());
+        // (without the accumulators the launch is simply not split)
+        if (r.ksplit > 1 && (!workspace || workspace_bytes < static_cast<size_t>(M) * N * sizeof(unsigned long long) ||
+                             reinterpret_cast<uintptr_t>(workspace) % 8 != 0))
+            r.ksplit = 1;
+        r.acc = static_cast<unsigned long long *>(workspace);
+        if (env_switches().show_plan)
+            fprintf(stderr, "sbvr_hip table look-up rows kernel M=%d N=%d K=%d S=%d: blocks=%d ksplit=%d\n", M, N, K, S, (N + 31) / 32, r.ksplit);
+        const hipError_t e = launch_rows32_lut(S, r, st);
+        if (e != hipSuccess)
+            return fail(SBVR_HIP_ELAUNCH, "rows32 (table look-up) launch: %s", hipGetErrorString(e));
+        g_last_kernel = SBVR_HIP_KERNEL_ROWS32;
+        return SBVR_HIP_OK;
     }
     if (pro.mode == kXPlain && !(flags & 3) && aligned && rows32_preferred(M, N, K, S, G, current_cus()) && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
         RowsArgs r{};
