@@ -2102,14 +2102,18 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
         uint32_t c[CW];
     };
     // (loads are never conditional: a pair past the range repeats the last one of K and is not computed)
-    auto load_line = [&](int ip) __attribute__((always_inline)) -> int {
+    // The two bytes of a line index stay as they were loaded until the step that uses them: any arithmetic on them
+    // here (even putting them into one word) would have to wait for them, and with them for every load issued before.
+    struct Line {
+        int lo, hi;
+    };
+    auto load_line = [&](int ip) __attribute__((always_inline)) -> Line {
         const int word = 2 * min(ip, pairs - 1);
         const size_t at = (static_cast<size_t>(word / a.words_per_group) * N + n_ld) << a.idx16;
         const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
-        const int lo = ib[at], hi = ib[at + a.idx16];          // two byte loads whatever the width: no branch
-        return lo | (hi << 16);
+        return Line{ib[at], ib[at + a.idx16]};                 // two byte loads whatever the width: no branch
     };
-    auto load_step = [&](int ip, Step &st, int line) __attribute__((always_inline)) {
+    auto load_step = [&](int ip, Step &st, const Line &line) __attribute__((always_inline)) {
         const int word = 2 * min(ip, pairs - 1) + h;
         const Planes<S> pl = load_planes<S, true>(a.bvr + (static_cast<size_t>(word) * N + n_ld) * S);
 #pragma unroll
@@ -2119,7 +2123,7 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             st.x[i] = xp[i];
-        const int ln = min(a.idx16 ? (line & 0xff) | ((line >> 8) & 0xff00) : line & 0xff, a.L - 1);
+        const int ln = min(a.idx16 ? line.lo | (line.hi << 8) : line.lo, a.L - 1);
         load_line_coeffs<S>(a.cache + static_cast<size_t>(ln) * S, st.c);
     };
 
@@ -2211,17 +2215,23 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
 
     // (two register sets: with three, the loads two steps ahead, the kernel needs 115 registers and was 8-25 % slower)
     Step s0, s1;
-    int line = load_line(p_begin);
+    Line line = load_line(p_begin);
     load_step(p_begin, s0, line);
     line = load_line(p_begin + 1);
+    // (the fences keep the loads of the next step in front of this step's arithmetic: left alone, the scheduler
+    // moves them down to their first use, to save registers, and every step waits for loads it has just issued)
     for (int ip = p_begin; ip < p_end; ip += 2) {
         load_step(ip + 1, s1, line);
         line = load_line(ip + 2);
+        __builtin_amdgcn_sched_barrier(0);
         compute(s0);
+        __builtin_amdgcn_sched_barrier(0);
         load_step(ip + 2, s0, line);
         line = load_line(ip + 3);
+        __builtin_amdgcn_sched_barrier(0);
         if (ip + 1 < p_end)
             compute(s1);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- partial results meet in LDS; D[i][jj] sits in lane jj + 32*((i/4)%2), register (i%4) + 4*(i/8)
