@@ -41,8 +41,8 @@ const char *sbvr_hip_last_error(void);
  * the routing depends on the shape and on the device (see sbvr_hip_linear_f16), and the kernels differ in
  * how they round, so a caller or a test that cares can ask. */
 #define SBVR_HIP_KERNEL_PORTABLE 1       /* one thread per output */
-#define SBVR_HIP_KERNEL_DECODE 2         /* up to 16 rows, plane sums on the matrix cores, exact activations */
-#define SBVR_HIP_KERNEL_ROWS32 3         /* up to 32 rows, weights decoded to fp16 in registers */
+#define SBVR_HIP_KERNEL_DECODE 2         /* up to 16 rows (8 by default), plane sums on the matrix cores, exact activations */
+#define SBVR_HIP_KERNEL_ROWS32 3         /* up to 32 rows (9..32 by default), weights decoded to fp16 in registers */
 #define SBVR_HIP_KERNEL_PREFILL 4        /* weights decoded to fp16 tiles in LDS */
 #define SBVR_HIP_KERNEL_PREFILL_SPLIT 5  /* the same with K split across workgroups (workspace given) */
 int sbvr_hip_last_kernel(void);
@@ -54,10 +54,11 @@ int sbvr_hip_init(int device);
 /* Bytes of device workspace sbvr_hip_linear_f16 wants for this shape (0 if
  * none).  The workspace must be zero-filled once after allocation; every call
  * leaves it zero-filled.  Calls that share a workspace must not overlap in
- * time.  For up to 16 rows (decode kernel, K split across workgroups) the
- * workspace is required; for more rows (prefill kernel with few output tiles)
- * it is optional: without it that launch is not split along K, which is slower
- * but gives the same result up to the order of the fp32 additions. */
+ * time.  Where the decode kernel splits K across workgroups the workspace is
+ * required; for the 32-row kernel with few columns and the prefill kernel with
+ * few output tiles it is optional: without it that launch is not split along K,
+ * which is slower but gives the same result up to the order of the fp32
+ * additions. */
 size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
 
 /*
@@ -78,17 +79,21 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  *   decode kernel   M <= 16, N >= 16, K and G multiples of 128 with G/128 a power
  *                   of two, S in {2,3,4,6,8}: plane sums on the matrix cores over
  *                   the raw bit planes, the fp16 activations represented exactly;
- *                   within 2 fp16 ulps of the exact sum.  Taken for every M <= 16
- *                   of such a shape (5..16 rows in a variant whose waves share the
+ *                   within 2 fp16 ulps of the exact sum.  Taken for up to 8 rows
+ *                   of such a shape, and for 9..16 rows where the 32-row kernel's
+ *                   table look-up form has no instance (6 or 8 planes) or flags
+ *                   bit 1 is set (5..16 rows in a variant whose waves share the
  *                   activation operands, where N >= 32 for up to 8 rows, 64 beyond);
- *   32-row kernel   5 <= M <= 32, K and G multiples of 32, same S: taken for
- *                   17..32 rows, and for 5..16 rows of shapes the decode kernel
- *                   does not cover (N < 16, K or G not a multiple of 128).  For
- *                   17..32 rows with 2, 3 or 4 planes and K and G multiples of 64
- *                   it decodes by table look-up (the subset sums of a group's
- *                   coefficient line) and, with a workspace and few columns,
- *                   splits K across workgroups through the decode kernel's
- *                   accumulators; same results as its arithmetic form;
+ *   32-row kernel   up to 32 rows.  Its table look-up form (2, 3 or 4 planes, K and
+ *                   G multiples of 64: a weight is looked up among the subset sums
+ *                   of its group's coefficient line; with a workspace and few
+ *                   columns K is split across workgroups through the decode
+ *                   kernel's accumulators) is taken for 9..32 rows: from 9 rows on
+ *                   it is the faster one (4096 -> 14336, 4 planes, 16 rows: 15.4 us
+ *                   against 20 us).  Its arithmetic form (K and G multiples of 32,
+ *                   S in {2,3,4,6,8}; same results) takes 17..32 rows otherwise, and
+ *                   5..16 rows of shapes the decode kernel does not cover (N < 16,
+ *                   K or G not a multiple of 128);
  *   prefill kernel  M > 32 (or 17..32 with flags bit 1), K and G multiples of 64,
  *                   same S; with a workspace and few output tiles, K is split
  *                   across workgroups;
@@ -102,7 +107,8 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  * trans=True layout); this is the operator its models/sbvr_llama.py:86-87
  * SBVRLinear.forward stands for.
  * flags: bit 0 forces the portable kernel; bit 1 keeps the 32-row kernel out
- * (5..16 rows then take the decode kernel, 17..32 the prefill kernel).
+ * (5..16 rows then take the decode kernel, exact in weights and activations,
+ * 17..32 the prefill kernel).
  * Range: where the decode kernel splits K across workgroups, a workgroup's
  * partial sum is clamped to +-130000 before it is added up in fixed point;
  * partial sums beyond twice the fp16 range that would cancel to a finite total
@@ -119,10 +125,10 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
  * a workspace (code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc).  It has no counterpart in the reference.  Same
  * arguments and results as sbvr_hip_linear_f16 without the workspace pair: the
- * decode kernel's split-K accumulators live in a 4 MiB array inside the
- * library (one copy per GPU, held until the process ends), so up to 16 rows
- * need M * N <= 524288 (SBVR_HIP_EWORKSPACE beyond that); with more rows the
- * prefill kernel runs without its optional workspace, i.e. not split along K.
+ * split-K accumulators of the decode and 32-row kernels live in a 4 MiB array
+ * inside the library (one copy per GPU, held until the process ends), so up to
+ * 32 rows need M * N <= 524288 (SBVR_HIP_EWORKSPACE beyond that); with more rows
+ * the prefill kernel runs without its optional workspace, i.e. not split along K.
  * The call allocates and frees nothing.  Calls that overlap in time on one GPU
  * share the array and race: serialise them (one stream, or events).
  */

@@ -1,8 +1,8 @@
 // libsbvr_hip.so -- HIP kernels for gfx950 (MI355X) behind the C ABI of
 // include/sbvr_hip.h: the SBVR compressed-domain linear layer.
 //
-// Decode path (M <= 16), sbvr_gemv_mfma_kernel (and, for 5..16 rows, sbvr_gemv_batch_kernel, whose waves share
-// the activation operands of a sub-group).  The work is one bit per weight
+// Decode path (M <= 8 by default, M <= 16 on request and with 6 or 8 planes), sbvr_gemv_mfma_kernel (and, from
+// 5 rows on, sbvr_gemv_batch_kernel, whose waves share the activation operands of a sub-group).  The work is one bit per weight
 // element and plane, far too many bits for one VALU lane-op each, so the masked
 // sums run on the matrix cores:
 //   * a 32-bit plane word becomes four dwords of fp4 (e2m1) values with one AND
@@ -31,9 +31,10 @@
 // activations into A operands: sbvr_hip_linear_f16_swiglu / _add_rmsnorm.
 //
 // Prefill path (M > 32), sbvr_gemm_mfma_kernel: weights decoded to fp16 tiles
-// in LDS, fp16 MFMA, fp32 accumulation; sbvr_gemm_rows32_kernel for 17..32 rows
-// (the batch rows are the 32 rows of one MFMA, weights decoded in registers;
-// sbvr_gemm_rows32_lut_kernel decodes them by table look-up for 2..4 planes).
+// in LDS, fp16 MFMA, fp32 accumulation.  In between, 9..32 rows (17..32 with 6
+// or 8 planes): the batch rows are the 32 rows of one MFMA, weights decoded in
+// registers -- by table look-up for 2..4 planes (sbvr_gemm_rows32_lut_kernel),
+// arithmetically otherwise (sbvr_gemm_rows32_kernel).
 //
 // The reference's own operator forms: both operands encoded: the decode kernel
 // with the left operand's planes as batch rows (one left row of up to 4 planes),
@@ -2022,10 +2023,8 @@ bool rows32_path_ok(int M, int N, int K, int S, int G)
            static_cast<double>(K / 32) * N * S < 2147483648.0;
 }
 
-// Measured on MI355X at the Llama-3-8B shapes: the 32-row kernel takes about the same
-// time for any batch up to 32 (24-25 us at 4096 -> 14336), the decode kernels 13 us at 8 rows
-// and 21 us at 16: the 32-row kernel is for 17..32 rows, and for 5..16 rows of shapes the
-// decode kernels do not cover.
+// The arithmetic form of the 32-row kernel: for 17..32 rows where the table look-up form has no instance (6 or 8
+// planes, K or G not a multiple of 64), and for 5..16 rows of shapes the decode kernels do not cover.
 bool rows32_preferred(int M, int N, int K, int S, int G, int cus)
 {
     (void)cus;
@@ -2074,14 +2073,24 @@ hipError_t launch_rows32(int S, RowsArgs a, hipStream_t st)
 // 64 bytes, four loads) are put into that order with four permutes per MFMA.
 // K can be split across workgroups (blockIdx.y) through the decode kernel's 64-bit accumulators.
 constexpr int kLutWaves = 8;
-constexpr int kLutMinRows = 17;      // batch rows from which the linear takes this kernel
+// Batch rows from which the linear takes this kernel.  Measured at 4096 -> 14336 / 14336 -> 4096, 4 planes: 15.3-16.1 us
+// for any row count up to 16 (17.3-17.5 at 32; 11.4-12.5 with 2 planes, 12.6-13.7 with 3), against 11.7-12.5 us at
+// 5..8 rows and 17.9-20.9 us at 9..16 rows for the decode kernels (13.6-16.0 with 2 planes, 19.6-22.5 with 3).
+constexpr int kLutMinRows = 9;
 
-template <int S>
+// kHalfRows: up to 16 batch rows (the activation loads of rows 16..31 are left out); kShare: groups of a multiple
+// of 128 elements, so the two steps of a loop iteration (an even word pair and the next) share a coefficient line:
+// one index load, one gather and one table per two steps.
+template <int S, bool kHalfRows, bool kShare>
 __global__ void __launch_bounds__(64 * kLutWaves)
 sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
 {
     static_assert(S >= 2 && S <= 4, "tables of 4, 8 or 16 entries");
     __shared__ float red[kLutWaves][16][64];
+    // a wave's activations of one step: 32 rows of 128 bytes (the word pair), rows 144 bytes apart so that 16 lanes
+    // reading the same 16-byte chunk of 16 rows hit 16 different bank groups
+    constexpr int kXRow = 144;
+    __shared__ __align__(16) unsigned char xs[kLutWaves][32 * kXRow];
     constexpr int CW = (S + 1) / 2;
     constexpr int TW = S == 4 ? 4 : (S == 3 ? 2 : 1);       // dwords of a byte table
 
@@ -2092,9 +2101,18 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
     const int n = blockIdx.x * 32 + j, n_ld = min(n, N - 1);
     const int pairs = K / 64;
     const int wg_begin = blockIdx.y * a.pairs_per_wg, wg_end = min(pairs, wg_begin + a.pairs_per_wg);
-    const int ppw = (wg_end - wg_begin + kLutWaves - 1) / kLutWaves;
+    const int ppw = ((wg_end - wg_begin + kLutWaves - 1) / kLutWaves + 1) / 2 * 2;     // even: see the loop
     const int p_begin = wg_begin + wave * ppw, p_end = min(wg_end, p_begin + ppw);
-    const uint16_t *xrow = a.x + static_cast<size_t>(min(j, M - 1)) * K + 32 * h;      // (rows past M repeat the last one; dropped at the end)
+    // The activations come in whole cache lines: load i of a step brings rows 8i .. 8i+7, eight lanes per row (128
+    // bytes: the 64 elements of the word pair), and goes through LDS to the lanes that want a row each.  (A lane
+    // loading its own row's 64 bytes touches 64 cache lines per load instruction; the launch was bound by that.)
+    const uint16_t *xsrc = a.x + 8 * (lane & 7);
+    size_t xoff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        xoff[i] = static_cast<size_t>(min(8 * i + (lane >> 3), M - 1)) * K;     // (rows past M repeat the last one; dropped at the end)
+    unsigned char *const xw = xs[wave] + (lane >> 3) * kXRow + (lane & 7) * 16;  // + 8 i rows
+    const unsigned char *const xr = xs[wave] + j * kXRow + 64 * h;                // this lane's row, its word's 64 bytes
 
     struct Step {
         uint32_t w[S];
@@ -2113,18 +2131,19 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
         const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
         return Line{ib[at], ib[at + a.idx16]};                 // two byte loads whatever the width: no branch
     };
-    auto load_step = [&](int ip, Step &st, const Line &line) __attribute__((always_inline)) {
+    auto load_step = [&](int ip, Step &st, const Line &line, bool with_line) __attribute__((always_inline)) {
         const int word = 2 * min(ip, pairs - 1) + h;
         const Planes<S> pl = load_planes<S, true>(a.bvr + (static_cast<size_t>(word) * N + n_ld) * S);
 #pragma unroll
         for (int q = 0; q < S; ++q)
             st.w[q] = pl.w[q];
-        const v4u *xp = reinterpret_cast<const v4u *>(xrow + 64 * min(ip, pairs - 1));
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            st.x[i] = xp[i];
-        const int ln = min(a.idx16 ? line.lo | (line.hi << 8) : line.lo, a.L - 1);
-        load_line_coeffs<S>(a.cache + static_cast<size_t>(ln) * S, st.c);
+        for (int i = 0; i < (kHalfRows ? 2 : 4); ++i)
+            st.x[i] = *reinterpret_cast<const v4u *>(xsrc + xoff[i] + 64 * min(ip, pairs - 1));
+        if (with_line) {                  // (known where the call is written: no branch)
+            const int ln = min(a.idx16 ? line.lo | (line.hi << 8) : line.lo, a.L - 1);
+            load_line_coeffs<S>(a.cache + static_cast<size_t>(ln) * S, st.c);
+        }
     };
 
     v16f acc;
@@ -2135,16 +2154,17 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
     auto rotr = [](uint32_t v, int r) __attribute__((always_inline)) -> uint32_t {
         return (r & 31) == 0 ? v : __builtin_amdgcn_alignbit(v, v, r & 31);
     };
-    auto compute = [&](const Step &st) __attribute__((always_inline)) {
-        // ---- the group's subset sums, entries (2i, 2i + 1) as packed pairs, then as byte tables
+    uint32_t tlo[TW], thi[TW];
+    // ---- the group's subset sums, entries (2i, 2i + 1) as packed pairs, then as byte tables
+    auto build_table = [&](const uint32_t (&c)[CW]) __attribute__((always_inline)) {
         v2h cc[S];
 #pragma unroll
         for (int q = 0; q < S; ++q) {
-            const uint32_t bits = q & 1 ? st.c[q / 2] >> 16 : st.c[q / 2] & 0xffffu;
+            const uint32_t bits = q & 1 ? c[q / 2] >> 16 : c[q / 2] & 0xffffu;
             cc[q] = as_v2h(bits | (bits << 16));
         }
         v2h e[1 << (S - 1)];
-        e[0] = as_v2h((st.c[0] & 0xffffu) << 16);             // entries 0, 1: nothing, c0
+        e[0] = as_v2h((c[0] & 0xffffu) << 16);                // entries 0, 1: nothing, c0
         e[1] = e[0] + cc[1];                                   // 2, 3
         if constexpr (S >= 3) {
             e[2] = e[0] + cc[2];                               // 4, 5
@@ -2155,13 +2175,24 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
             for (int i = 0; i < 4; ++i)
                 e[4 + i] = e[i] + cc[3];                       // 8..15: the last plane is added last
         }
-        uint32_t tlo[TW], thi[TW];
 #pragma unroll
         for (int i = 0; i < TW; ++i) {
             const uint32_t e0 = __builtin_bit_cast(uint32_t, e[2 * i]), e1 = __builtin_bit_cast(uint32_t, e[2 * i + 1]);
             tlo[i] = __builtin_amdgcn_perm(e1, e0, 0x06040200u);
             thi[i] = __builtin_amdgcn_perm(e1, e0, 0x07050301u);
         }
+    };
+    auto compute = [&](const Step &st) __attribute__((always_inline)) {
+        // ---- activations: rows as loaded -> LDS -> a row per lane (the LDS serves a wave's accesses in order)
+#pragma unroll
+        for (int i = 0; i < (kHalfRows ? 2 : 4); ++i)
+            *reinterpret_cast<v4u *>(xw + 8 * i * kXRow) = st.x[i];
+        __builtin_amdgcn_wave_barrier();
+        v4u xl[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            xl[i] = *reinterpret_cast<const v4u *>(xr + 16 * i);
+        __builtin_amdgcn_wave_barrier();
         // ---- nibble words: nibble n of Q[p] = selector of element p + 4n
         uint32_t Q[4];
 #pragma unroll
@@ -2204,7 +2235,7 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
             const v4u bw = {b0, b1, b2, b3};
             v4u aw;
             // dword i of the lane's 64 bytes of activations holds elements 2i, 2i + 1
-            const uint32_t d0 = st.x[0][q], d1 = st.x[1][q], d2 = st.x[2][q], d3 = st.x[3][q];
+            const uint32_t d0 = xl[0][q], d1 = xl[1][q], d2 = xl[2][q], d3 = xl[3][q];
             aw.x = __builtin_amdgcn_perm(d1, d0, 0x05040100u);
             aw.y = __builtin_amdgcn_perm(d3, d2, 0x05040100u);
             aw.z = __builtin_amdgcn_perm(d1, d0, 0x07060302u);
@@ -2216,21 +2247,26 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
     // (two register sets: with three, the loads two steps ahead, the kernel needs 115 registers and was 8-25 % slower)
     Step s0, s1;
     Line line = load_line(p_begin);
-    load_step(p_begin, s0, line);
-    line = load_line(p_begin + 1);
+    load_step(p_begin, s0, line, true);
+    line = load_line(p_begin + (kShare ? 2 : 1));
     // (the fences keep the loads of the next step in front of this step's arithmetic: left alone, the scheduler
     // moves them down to their first use, to save registers, and every step waits for loads it has just issued)
     for (int ip = p_begin; ip < p_end; ip += 2) {
-        load_step(ip + 1, s1, line);
-        line = load_line(ip + 2);
+        load_step(ip + 1, s1, line, !kShare);
+        if constexpr (!kShare)
+            line = load_line(ip + 2);
         __builtin_amdgcn_sched_barrier(0);
+        build_table(s0.c);
         compute(s0);
         __builtin_amdgcn_sched_barrier(0);
-        load_step(ip + 2, s0, line);
-        line = load_line(ip + 3);
+        load_step(ip + 2, s0, line, true);
+        line = load_line(ip + (kShare ? 4 : 3));
         __builtin_amdgcn_sched_barrier(0);
-        if (ip + 1 < p_end)
+        if (ip + 1 < p_end) {
+            if constexpr (!kShare)
+                build_table(s1.c);
             compute(s1);
+        }
         __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -2291,17 +2327,31 @@ int lut_ksplit(int N, int K, int cus)
 
 hipError_t launch_rows32_lut(int S, RowsArgs a, hipStream_t st)
 {
+    // (an even number of word pairs per workgroup and per wave: a loop iteration starts on an even pair, which the
+    // shared coefficient line of the kShare instances relies on)
     const int pairs = a.K / 64;
-    a.pairs_per_wg = (pairs + a.ksplit - 1) / a.ksplit;
+    a.pairs_per_wg = ((pairs + a.ksplit - 1) / a.ksplit + 1) / 2 * 2;
     const dim3 grid(static_cast<unsigned>((a.N + 31) / 32), static_cast<unsigned>(a.ksplit)), block(64 * kLutWaves);
+    const bool half = a.M <= 16, share = a.words_per_group % 4 == 0;
+#define SBVR_LUT(SS)                                                                                          \
+    if (half && share)                                                                                        \
+        hipLaunchKernelGGL((sbvr_gemm_rows32_lut_kernel<SS, true, true>), grid, block, 0, st, a);             \
+    else if (half)                                                                                            \
+        hipLaunchKernelGGL((sbvr_gemm_rows32_lut_kernel<SS, true, false>), grid, block, 0, st, a);            \
+    else if (share)                                                                                           \
+        hipLaunchKernelGGL((sbvr_gemm_rows32_lut_kernel<SS, false, true>), grid, block, 0, st, a);            \
+    else                                                                                                      \
+        hipLaunchKernelGGL((sbvr_gemm_rows32_lut_kernel<SS, false, false>), grid, block, 0, st, a);           \
+    break
     switch (S) {
-    case 4: hipLaunchKernelGGL(sbvr_gemm_rows32_lut_kernel<4>, grid, block, 0, st, a); break;
+    case 4: SBVR_LUT(4);
 #ifndef SBVR_FAST_BUILD
-    case 2: hipLaunchKernelGGL(sbvr_gemm_rows32_lut_kernel<2>, grid, block, 0, st, a); break;
-    case 3: hipLaunchKernelGGL(sbvr_gemm_rows32_lut_kernel<3>, grid, block, 0, st, a); break;
+    case 2: SBVR_LUT(2);
+    case 3: SBVR_LUT(3);
 #endif
     default: return hipErrorInvalidConfiguration;
     }
+#undef SBVR_LUT
     return hipGetLastError();
 }
 
@@ -3293,14 +3343,14 @@ int sbvr_hip_linear_f16_noalloc(const void *x, const uint32_t *bvr, const void *
                                 void *out, int M, int N, int K, int S, int G, int L,
                                 int flags, void *stream)
 {
-    // The decode kernel's accumulators come from the library's own scratch array; the prefill kernel runs
-    // without its optional workspace (not split along K).  Nothing is allocated or freed on the way.
+    // The accumulators of the decode and 32-row kernels come from the library's own scratch array; the prefill
+    // kernel runs without its optional workspace (not split along K).  Nothing is allocated or freed on the way.
     void *ws = nullptr;
     size_t ws_bytes = 0;
-    if (M >= 1 && N >= 1 && mfma_path_ok(M, N, K, S, G) && !(flags & 1)) {
+    if (M >= 1 && N >= 1 && (mfma_path_ok(M, N, K, S, G) || lut_path_ok(M, N, K, S, G)) && !(flags & 1)) {
         const size_t need = static_cast<size_t>(M) * N * sizeof(unsigned long long);
         if (need > kScratchBytes)
-            return fail(SBVR_HIP_EWORKSPACE, "sbvr_hip_linear_f16_noalloc takes M * N <= %zu for up to 16 rows (M=%d N=%d); "
+            return fail(SBVR_HIP_EWORKSPACE, "sbvr_hip_linear_f16_noalloc takes M * N <= %zu for up to 32 rows (M=%d N=%d); "
                         "use sbvr_hip_linear_f16 with a workspace", kScratchBytes / sizeof(unsigned long long), M, N);
         const int rc = scratch_on_current_device(&ws);
         if (rc != SBVR_HIP_OK)

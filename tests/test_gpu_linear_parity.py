@@ -29,9 +29,24 @@ def check(y_gpu, yd, what=""):
     return rel.max(), ulp.max()
 
 
+def check_rounded(y_gpu, yd, what=""):
+    """The 32-row kernel (9..32 rows by default) rounds each decoded weight to fp16, as the reference's decode()
+    does: at most 3e-3 of the RMS output off, 1e-2 relative for outputs above 0.3 RMS."""
+    y = y_gpu.float().cpu().numpy().astype(np.float64)
+    rms = float(np.sqrt(np.mean(yd ** 2))) + 1e-30
+    err = np.abs(y - yd)
+    assert err.max() <= 3e-3 * rms + 2.0 ** -11 * np.abs(yd).max(), f"{what}: error {err.max() / rms:.3e} of the RMS output"
+    assert (err / np.maximum(np.abs(yd), 0.3 * rms)).max() <= 1e-2, what
+
+
+DECODE, ROWS32 = 2, 3
+
+
 def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False, flags=0, sigma=0.02, xscale=1.0):
+    """flags = 2 keeps the 32-row kernel out: 9..16 rows then take the decode kernel of 5..16 rows, which the
+    default dispatch uses up to 8 rows (and for 6 and 8 planes)."""
     import sbvr
-    from sbvr import synth
+    from sbvr import hip, synth
     dev = _dev()
     bvr, idx, cache = synth.random_encoding(N, K, S, G, L, sigma=sigma, seed=seed)
     gen = torch.Generator().manual_seed(seed + 1)
@@ -40,6 +55,9 @@ def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False, flags=0, sigma=0.02, 
     y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev),
                               None if b is None else b.to(dev), bvr_len=G, flags=flags)
     torch.cuda.synchronize()
+    ran = hip.last_kernel()
+    if flags == 2 and M <= 16:
+        assert ran != ROWS32 or G % 128 != 0 or N < 16, f"flags=2 ran kernel {ran}"
     yref, yd = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), G,
                                    None if b is None else b.numpy())
     if b is not None:
@@ -49,6 +67,8 @@ def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False, flags=0, sigma=0.02, 
         diff = np.abs(y.float().cpu().numpy().astype(np.float64) - yd)
         assert diff.max() <= 2.0 ** -9 * max(np.abs(yd).max(), rms), f"bias case off by {diff.max()}"
         return
+    if ran == ROWS32:
+        return check_rounded(y, yd, f"N={N} K={K} S={S} G={G} M={M} L={L} flags={flags} (32-row kernel)")
     return check(y, yd, f"N={N} K={K} S={S} G={G} M={M} L={L} flags={flags}")
 
 
@@ -109,39 +129,50 @@ def test_sweep_down(oracle, S, M):
     run_case(oracle, 4096, 14336, S, 128, M, 256, seed=14)
 
 
-def test_sweep_down_16_rows(oracle):
-    """16 rows at the down shape: four row tiles, K split 14 ways through the accumulators."""
-    run_case(oracle, 4096, 14336, 4, 128, 16, 256, seed=15)
+@pytest.mark.parametrize("flags", [0, 2])
+def test_sweep_down_16_rows(oracle, flags):
+    """16 rows at the down shape.  Default: the 32-row kernel, K in two parts.  flags = 2: the decode kernel, four
+    row tiles, K split 14 ways through the accumulators."""
+    run_case(oracle, 4096, 14336, 4, 128, 16, 256, seed=15, flags=flags)
 
 
-@pytest.mark.parametrize("M", [5, 6, 7, 8, 9, 12, 13, 16])
+@pytest.mark.parametrize("S", [2, 3, 4])
+def test_sweep_gate_16_rows_decode_kernel(oracle, S):
+    run_case(oracle, 14336, 4096, S, 128, 16, 256, seed=12, flags=2)
+
+
+@pytest.mark.parametrize("M,flags", [(5, 0), (6, 0), (7, 0), (8, 0), (9, 0), (9, 2), (12, 0), (12, 2), (13, 0), (13, 2),
+                                     (16, 0), (16, 2)])
 @pytest.mark.parametrize("N", [32, 48, 64, 100, 1000, 1030])
-def test_batch_rows_ragged_n(oracle, M, N):
+def test_batch_rows_ragged_n(oracle, M, N, flags):
     """5..16 rows: the waves of a workgroup share the activation operands of a sub-group and split its
     columns.  Windows that end inside a tile, windows moved left at the edge of N, and (N below 64 with more
     than 8 rows) the shapes that fall back to one wave per sub-group."""
     from sbvr import hip
-    run_case(oracle, N, 512, 4, 128, M, 64, seed=300 + M + N)
-    assert hip.last_kernel() == 2
+    run_case(oracle, N, 512, 4, 128, M, 64, seed=300 + M + N, flags=flags)
+    assert hip.last_kernel() == (DECODE if M <= 8 or flags == 2 else ROWS32)
 
 
+@pytest.mark.parametrize("flags", [0, 2])
 @pytest.mark.parametrize("S", [2, 3, 6, 8])
 @pytest.mark.parametrize("M", [7, 11])
-def test_batch_rows_planes(oracle, S, M):
-    run_case(oracle, 384, 1024, S, 128, M, 200, seed=320 + S + M)
+def test_batch_rows_planes(oracle, S, M, flags):
+    run_case(oracle, 384, 1024, S, 128, M, 200, seed=320 + S + M, flags=flags)
 
 
+@pytest.mark.parametrize("flags", [0, 2])
 @pytest.mark.parametrize("G", [128, 256, 512])
 @pytest.mark.parametrize("M", [8, 16])
-def test_batch_rows_groups(oracle, G, M):
-    run_case(oracle, 512, 2048, 4, G, M, 256, seed=340 + G + M)
+def test_batch_rows_groups(oracle, G, M, flags):
+    run_case(oracle, 512, 2048, 4, G, M, 256, seed=340 + G + M, flags=flags)
 
 
-def test_batch_rows_u16_index_bias_and_scales(oracle):
-    run_case(oracle, 320, 768, 4, 128, 6, 3000, seed=350)
-    run_case(oracle, 320, 768, 3, 128, 14, 5000, seed=351, bias=True)
-    run_case(oracle, 320, 768, 4, 128, 10, 256, seed=352, xscale=100.0)
-    run_case(oracle, 320, 768, 4, 128, 5, 256, seed=353, xscale=1e-3)
+@pytest.mark.parametrize("flags", [0, 2])
+def test_batch_rows_u16_index_bias_and_scales(oracle, flags):
+    run_case(oracle, 320, 768, 4, 128, 6, 3000, seed=350, flags=flags)
+    run_case(oracle, 320, 768, 3, 128, 14, 5000, seed=351, bias=True, flags=flags)
+    run_case(oracle, 320, 768, 4, 128, 10, 256, seed=352, xscale=100.0, flags=flags)
+    run_case(oracle, 320, 768, 4, 128, 5, 256, seed=353, xscale=1e-3, flags=flags)
 
 
 def test_batch_rows_of_different_magnitude(oracle):
@@ -157,13 +188,15 @@ def test_batch_rows_of_different_magnitude(oracle):
     x[5] = 0.0
     x[9] *= 1e-3
     x = x.to(torch.float16)
-    y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev), None, bvr_len=G)
     _, yd = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), G)
-    for m in range(M):           # row by row: each against its own RMS
-        if m == 5:
-            assert float(y[m].float().abs().max()) == 0.0
-        else:
-            check(y[m:m + 1], yd[m:m + 1], f"row {m}")
+    # flags = 2: the decode kernel of 5..16 rows (exact); default: the 32-row kernel (weights rounded to fp16)
+    for flags, judge in ((2, check), (0, check_rounded)):
+        y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev), None, bvr_len=G, flags=flags)
+        for m in range(M):           # row by row: each against its own RMS
+            if m == 5:
+                assert float(y[m].float().abs().max()) == 0.0
+            else:
+                judge(y[m:m + 1], yd[m:m + 1], f"row {m}, flags {flags}")
 
 
 def test_batch_rows_repeatable(oracle):
@@ -174,10 +207,11 @@ def test_batch_rows_repeatable(oracle):
     N, K, M = 1024, 4096, 16
     bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(N, K, 4, 128, 256, seed=370))
     x = torch.randn((M, K), generator=torch.Generator().manual_seed(371)).to(torch.float16).to(dev)
-    first = sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, bvr_len=128)
-    for _ in range(5):
-        again = sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, bvr_len=128)
-        assert torch.equal(first, again)
+    for flags in (2, 0):         # the decode kernel of 5..16 rows; the 32-row kernel, K in two parts
+        first = sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, bvr_len=128, flags=flags)
+        for _ in range(5):
+            again = sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, bvr_len=128, flags=flags)
+            assert torch.equal(first, again)
 
 
 def test_portable_kernel(oracle):
