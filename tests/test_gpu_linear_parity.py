@@ -5,7 +5,11 @@ Tolerance (fp16 outputs, fp32 accumulation): every output must lie within
 1e-2 relative of the oracle's unrounded double sum, outputs whose magnitude is
 below 1 % of the output RMS being judged against that RMS instead; on top of
 that the worst error must stay below 2 fp16 ulps of max(|ref|, RMS), which is
-what an fp32-accumulating kernel is expected to reach."""
+what an fp32-accumulating kernel is expected to reach.  (9 rows and more take
+the 32-row kernel by default, which rounds decoded weights to fp16: those runs
+are held to that kernel's bound, see check_rounded; flags = 2 keeps the decode
+kernel.)  The largest shapes are checked on a seeded sample of columns, the
+window edges always among them: the oracle is exact per column."""
 import numpy as np
 import pytest
 import torch
@@ -58,8 +62,18 @@ def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False, flags=0, sigma=0.02, 
     ran = hip.last_kernel()
     if flags == 2 and M <= 16:
         assert ran != ROWS32 or G % 128 != 0 or N < 16, f"flags=2 ran kernel {ran}"
-    yref, yd = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), G,
-                                   None if b is None else b.numpy())
+    bn, inn, bb = bvr.numpy(), idx.numpy(), None if b is None else b.numpy()
+    if float(N) * K * M > 2.5e8:
+        # Columns are independent: the oracle on a seeded sample of them (the first and last columns and the
+        # columns around the window edges of the decode kernel always among them) is exact for those columns.
+        rng = np.random.default_rng(seed)
+        count = max(256, int(2.5e8 / (float(K) * M)))
+        edges = [c for e in (0, 56, 64, 112, 128, N - 128, N - 112, N - 64, N - 56, N) for c in (e - 1, e, e + 1) if 0 <= c < N]
+        cols = np.unique(np.concatenate([rng.choice(N, size=min(count, N), replace=False), np.array(edges, dtype=np.int64)]))
+        bn, inn = np.ascontiguousarray(bn[:, cols, :]), np.ascontiguousarray(inn[:, cols])
+        bb = None if bb is None else np.ascontiguousarray(bb[cols])
+        y = y[:, torch.from_numpy(cols).to(y.device)]
+    yref, yd = oracle.C.linear_f16(x.numpy(), bn, inn, cache.numpy(), G, bb)
     if b is not None:
         # bias is added after rounding; judge the pre-bias part through the fp16 reference too
         yd = yref.astype(np.float64)
