@@ -96,7 +96,11 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  *                   K or G not a multiple of 128);
  *   prefill kernel  M > 32 (or 17..32 with flags bit 1), K and G multiples of 64,
  *                   same S; with a workspace and few output tiles, K is split
- *                   across workgroups;
+ *                   across workgroups.  With 2, 3 or 4 planes and K and G multiples
+ *                   of 128 it is the kernel that decodes by table look-up in
+ *                   registers (256 x 256 output tiles, the weights never in LDS),
+ *                   otherwise the one that decodes weight tiles into LDS; same
+ *                   results up to the order of the fp32 additions;
  *   portable kernel everything else (one thread per output), and with flags bit 0.
  * The 32-row and prefill kernels decode the weights to fp16 first (each decoded
  * weight an fp16 sum of its coefficients, as decode() of sbvr/core.py:927-949

@@ -30,8 +30,10 @@
 // linear along (SiLU(gate) * up, or residual add + RMSNorm) while it turns the
 // activations into A operands: sbvr_hip_linear_f16_swiglu / _add_rmsnorm.
 //
-// Prefill path (M > 32), sbvr_gemm_mfma_kernel: weights decoded to fp16 tiles
-// in LDS, fp16 MFMA, fp32 accumulation.  In between, 9..32 rows (17..32 with 6
+// Prefill path (M > 32): fp16 MFMA, fp32 accumulation; sbvr_gemm_lut_kernel (2..4
+// planes: weights decoded by table look-up in registers, activations shared
+// through LDS) or sbvr_gemm_mfma_kernel (weights decoded to fp16 tiles in LDS by
+// producer waves).  In between, 9..32 rows (17..32 with 6
 // or 8 planes): the batch rows are the 32 rows of one MFMA, weights decoded in
 // registers -- by table look-up for 2..4 planes (sbvr_gemm_rows32_lut_kernel),
 // arithmetically otherwise (sbvr_gemm_rows32_kernel).
@@ -1087,7 +1089,7 @@ struct GemvPlan {
 
 // Development switches, read from the environment once per process.
 struct EnvSwitches {
-    int ct, sp, waves, wstride, show_plan, popc_q, rowdeq_lanes, lut_rows;
+    int ct, sp, waves, wstride, show_plan, popc_q, rowdeq_lanes, lut_rows, pf_lut;
 };
 
 const EnvSwitches &env_switches()
@@ -1098,7 +1100,7 @@ const EnvSwitches &env_switches()
             return v && *v ? atoi(v) : 0;
         };
         return EnvSwitches{get("SBVR_HIP_CT"), get("SBVR_HIP_SP"), get("SBVR_HIP_WAVES"), get("SBVR_HIP_WSTRIDE"),
-                           get("SBVR_HIP_SHOW_PLAN"), get("SBVR_HIP_POPC_Q"), get("SBVR_HIP_ROWDEQ_LANES"), get("SBVR_HIP_LUT_ROWS")};
+                           get("SBVR_HIP_SHOW_PLAN"), get("SBVR_HIP_POPC_Q"), get("SBVR_HIP_ROWDEQ_LANES"), get("SBVR_HIP_LUT_ROWS"), get("SBVR_HIP_PF_LUT")};
     }();
     return e;
 }
@@ -2426,6 +2428,314 @@ hipError_t launch_gemm(int S, const GemmArgs &a, hipStream_t st)
     return hipGetLastError();
 }
 
+// ------------------------------------------- MFMA prefill with the weights decoded by table look-up
+//
+// The prefill contraction with the decode of sbvr_gemm_rows32_lut_kernel: no producer and consumer waves and no
+// weight tile in LDS.  A workgroup of 8 waves owns 256 rows x 256 columns of the output; wave w owns columns
+// 32w .. 32w+31 for all 256 rows (8 row blocks of 32: 128 accumulator registers a lane).  Per step of 64 elements
+// of K a lane (column j, half h) decodes its word 2i + h of column j by table look-up straight into the B operands
+// of four MFMAs (16 registers), and the wave runs them against the 8 row blocks: 32 MFMAs per 32 weights decoded
+// per lane, so the decode (about 170 VALU instructions a step) hides behind the matrix pipe (32 x 32 clocks).
+// The activations of a step, 256 rows x 64 elements, are shared by the 8 waves through LDS, stored in the element
+// order the MFMAs want (see sbvr_gemm_rows32_lut_kernel: that permutation is done once, by the thread that
+// brings a (row, word) in, not once per wave): rows 144 bytes apart, two buffers, one barrier per step.  The loads
+// of the step after the next one's (activations, plane words) are in flight while a step is computed.
+// 2, 3 or 4 planes, K and G multiples of 128 (the two steps of a loop iteration share a coefficient line).
+// K can be split across workgroups (blockIdx.z) as in sbvr_gemm_mfma_kernel: fp32 partial tiles, second pass.
+constexpr int kPfWaves = 8, kPfBM = 256, kPfBN = 256, kPfRow = 144;
+constexpr int kPfTile = kPfBM * kPfRow;
+
+template <int S>
+__global__ void __launch_bounds__(64 * kPfWaves)
+sbvr_gemm_lut_kernel(const GemmArgs a)
+{
+    static_assert(S >= 2 && S <= 4, "tables of 4, 8 or 16 entries");
+    extern __shared__ __align__(16) unsigned char psm[];
+    constexpr int CW = (S + 1) / 2;
+    constexpr int TW = S == 4 ? 4 : (S == 3 ? 2 : 1);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int N = a.N, K = a.K, M = a.M;
+    const int j = lane & 31, h = lane >> 5;
+    const int n0 = blockIdx.x * kPfBN, m0 = blockIdx.y * kPfBM;
+    const int n = n0 + 32 * wave + j, n_ld = min(n, N - 1);
+    const int steps = K / 64 / a.ksplit;                 // of this workgroup, even
+    const int p0 = blockIdx.z * steps, p_last = p0 + steps - 1;
+    const int wpg = 2 * a.steps_per_group;               // words per group
+
+    // bringing activations in: thread t takes (row t / 2, word t % 2) of a step, 64 bytes
+    const uint16_t *xsrc = a.x + static_cast<size_t>(min(m0 + (tid >> 1), M - 1)) * K + 32 * (tid & 1);
+    unsigned char *const xdst = psm + (tid >> 1) * kPfRow + (tid & 1) * 64;
+    const unsigned char *const xrd = psm + j * kPfRow + h * 64;      // + 32 rb rows, + 16 q
+
+    struct Line {
+        int lo, hi;
+    };
+    auto load_line = [&](int ip) __attribute__((always_inline)) -> Line {
+        const size_t at = (static_cast<size_t>((2 * min(ip, p_last)) / wpg) * N + n_ld) << a.idx16;
+        const uint8_t *ib = static_cast<const uint8_t *>(a.idx);
+        return Line{ib[at], ib[at + a.idx16]};
+    };
+    auto load_coefficients = [&](const Line &line, uint32_t (&c)[CW]) __attribute__((always_inline)) {
+        const int ln = min(a.idx16 ? line.lo | (line.hi << 8) : line.lo, a.L - 1);
+        load_line_coeffs<S>(a.cache + static_cast<size_t>(ln) * S, c);
+    };
+    auto load_words = [&](int ip, uint32_t (&w)[S]) __attribute__((always_inline)) {
+        const int word = 2 * min(ip, p_last) + h;
+        const Planes<S> pl = load_planes<S>(a.bvr + (static_cast<size_t>(word) * N + n_ld) * S);
+#pragma unroll
+        for (int q = 0; q < S; ++q)
+            w[q] = pl.w[q];
+    };
+    auto load_x = [&](int ip, v4u (&x)[4]) __attribute__((always_inline)) {
+        const v4u *xp = reinterpret_cast<const v4u *>(xsrc + 64 * min(ip, p_last));
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            x[i] = xp[i];
+    };
+    // the 32 elements of a (row, word), dword i = elements 2i, 2i + 1, into the order of the four MFMAs' A operands:
+    // operand q = elements 2q, 2q+8, 2q+16, 2q+24, 2q+1, 2q+9, 2q+17, 2q+25
+    auto store_x = [&](const v4u (&x)[4], int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t d0 = x[0][q], d1 = x[1][q], d2 = x[2][q], d3 = x[3][q];
+            v4u aw;
+            aw.x = __builtin_amdgcn_perm(d1, d0, 0x05040100u);
+            aw.y = __builtin_amdgcn_perm(d3, d2, 0x05040100u);
+            aw.z = __builtin_amdgcn_perm(d1, d0, 0x07060302u);
+            aw.w = __builtin_amdgcn_perm(d3, d2, 0x07060302u);
+            *reinterpret_cast<v4u *>(xdst + buf * kPfTile + 16 * q) = aw;
+        }
+    };
+
+    uint32_t tlo[TW], thi[TW];
+    auto build_table = [&](const uint32_t (&c)[CW]) __attribute__((always_inline)) {
+        v2h cc[S];
+#pragma unroll
+        for (int q = 0; q < S; ++q) {
+            const uint32_t bits = q & 1 ? c[q / 2] >> 16 : c[q / 2] & 0xffffu;
+            cc[q] = as_v2h(bits | (bits << 16));
+        }
+        v2h e[1 << (S - 1)];
+        e[0] = as_v2h((c[0] & 0xffffu) << 16);
+        e[1] = e[0] + cc[1];
+        if constexpr (S >= 3) {
+            e[2] = e[0] + cc[2];
+            e[3] = e[1] + cc[2];
+        }
+        if constexpr (S == 4) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                e[4 + i] = e[i] + cc[3];
+        }
+#pragma unroll
+        for (int i = 0; i < TW; ++i) {
+            const uint32_t e0 = __builtin_bit_cast(uint32_t, e[2 * i]), e1 = __builtin_bit_cast(uint32_t, e[2 * i + 1]);
+            tlo[i] = __builtin_amdgcn_perm(e1, e0, 0x06040200u);
+            thi[i] = __builtin_amdgcn_perm(e1, e0, 0x07050301u);
+        }
+    };
+
+    v16f acc[8];
+#pragma unroll
+    for (int rb = 0; rb < 8; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            acc[rb][r] = 0.f;
+
+    auto rotr = [](uint32_t v, int r) __attribute__((always_inline)) -> uint32_t {
+        return (r & 31) == 0 ? v : __builtin_amdgcn_alignbit(v, v, r & 31);
+    };
+    auto compute = [&](const uint32_t (&w)[S], int buf) __attribute__((always_inline)) {
+        uint32_t Q[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            uint32_t v = rotr(w[0], p) & 0x11111111u;
+            v = (rotr(w[1], p - 1) & 0x22222222u) | v;
+            if constexpr (S >= 3)
+                v = (rotr(w[2], p - 2) & 0x44444444u) | v;
+            if constexpr (S == 4)
+                v = (rotr(w[3], p - 3) & 0x88888888u) | v;
+            Q[p] = v;
+        }
+        auto look_up = [&](int p, uint32_t &w01, uint32_t &w23) __attribute__((always_inline)) {
+            const uint32_t qs = p < 4 ? Q[p & 3] : Q[p & 3] >> 4;
+            const uint32_t sel = qs & (S == 2 ? 0x03030303u : 0x07070707u);
+            uint32_t lo, hi;
+            if constexpr (S == 2) {
+                lo = __builtin_amdgcn_perm(tlo[0], tlo[0], sel);
+                hi = __builtin_amdgcn_perm(thi[0], thi[0], sel);
+            } else {
+                lo = __builtin_amdgcn_perm(tlo[1], tlo[0], sel);
+                hi = __builtin_amdgcn_perm(thi[1], thi[0], sel);
+            }
+            if constexpr (S == 4) {
+                const uint32_t upper = __builtin_amdgcn_perm(0x0000ff00u, 0x0000ff00u, (qs >> 3) & 0x01010101u);
+                const uint32_t lo_u = __builtin_amdgcn_perm(tlo[3], tlo[2], sel), hi_u = __builtin_amdgcn_perm(thi[3], thi[2], sel);
+                lo = (lo_u & upper) | (lo & ~upper);
+                hi = (hi_u & upper) | (hi & ~upper);
+            }
+            w01 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
+            w23 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
+        };
+        auto operand = [&](int q) __attribute__((always_inline)) -> v4u {
+            uint32_t b0, b1, b2, b3;
+            look_up(2 * q, b0, b1);
+            look_up(2 * q + 1, b2, b3);
+            return v4u{b0, b1, b2, b3};
+        };
+        // MFMA q of all 8 row blocks in a row (8 different accumulators), its 8 activation operands read while
+        // MFMA q - 1 runs, and the look-ups of operand q + 1 in the shadow of the matrix pipe
+        const unsigned char *xt = xrd + buf * kPfTile;
+        v4u A[2][8];
+        auto read_a = [&](int q, v4u (&dst)[8]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int rb = 0; rb < 8; ++rb)
+                dst[rb] = *reinterpret_cast<const v4u *>(xt + 32 * rb * kPfRow + 16 * q);
+        };
+        read_a(0, A[0]);
+        v4u Bq = operand(0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            v4u Bn = Bq;
+            if (q < 3) {
+                read_a(q + 1, A[(q + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                Bn = operand(q + 1);
+            }
+#pragma unroll
+            for (int rb = 0; rb < 8; ++rb)
+                acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, A[q & 1][rb]), __builtin_bit_cast(v8h, Bq), acc[rb], 0, 0, 0);
+            Bq = Bn;
+        }
+    };
+
+    // -- prologue: the first step's activations into buffer 0, everything of the second in flight
+    // (decoding a step's operands one step ahead, in the shadow of the step before's MFMAs, measured no faster)
+    uint32_t wa[S], wb[S], c[CW], c_next[CW];
+    v4u xa[4];
+    Line line = load_line(p0);
+    load_words(p0, wa);
+    load_x(p0, xa);
+    load_coefficients(line, c);
+    line = load_line(p0 + 2);
+    store_x(xa, 0);
+    load_x(p0 + 1, xa);
+    load_words(p0 + 1, wb);
+    __syncthreads();
+    for (int ip = p0; ip <= p_last; ip += 2) {
+        // -- even step: buffer 0
+        load_coefficients(line, c_next);              // of the next pair of steps
+        line = load_line(ip + 4);
+        __builtin_amdgcn_sched_barrier(0);
+        build_table(c);
+        compute(wa, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        store_x(xa, 1);                                // step ip + 1
+        load_x(ip + 2, xa);
+        load_words(ip + 2, wa);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        // -- odd step: buffer 1
+        compute(wb, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        store_x(xa, 0);                                // step ip + 2
+        load_x(ip + 3, xa);
+        load_words(ip + 3, wb);
+#pragma unroll
+        for (int q = 0; q < CW; ++q)
+            c[q] = c_next[q];
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+    }
+
+    // ---- D[i][jj] of a row block sits in lane jj + 32*((i/4)%2), register (i%4) + 4*(i/8)
+    if (a.ksplit > 1) {
+        float *mine = a.part + blockIdx.z * (static_cast<size_t>(M) * N);
+#pragma unroll
+        for (int rb = 0; rb < 8; ++rb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + 32 * rb + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (m < M && n < N)
+                    mine[static_cast<size_t>(m) * N + n] = acc[rb][r];
+            }
+        return;
+    }
+    if (n >= N)
+        return;
+    const uint16_t bias = a.bias ? a.bias[n] : 0;
+#pragma unroll
+    for (int rb = 0; rb < 8; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = m0 + 32 * rb + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (m < M) {
+                uint16_t v = f2h(acc[rb][r]);
+                if (a.bias)
+                    v = hadd(v, bias);
+                a.out[static_cast<size_t>(m) * N + n] = v;
+            }
+        }
+}
+
+bool gemm_lut_path_ok(int M, int N, int K, int S, int G)
+{
+    return M > kRowsMax && K % 128 == 0 && G % 128 == 0 && (S == 2 || S == 3 || S == 4) &&
+           static_cast<double>(K / 32) * N * S < 2147483648.0 && static_cast<double>(M) * K < 2147483648.0;
+}
+
+// Workgroups along K for the table look-up prefill kernel: until the 256 x 256 tiles times the parts give three
+// quarters of the chip's 256 CUs a workgroup, a part keeping 16 steps and more (an even number).  A function of the
+// shape only.  (8192 -> 28672: 112 tiles at 256 rows take 229-236 us unsplit and 187 us in two parts; 224 tiles at
+// 512 rows 293 us unsplit and 340 us in two parts.)
+int gemm_lut_ksplit(int M, int N, int K)
+{
+    const int tiles = ((N + kPfBN - 1) / kPfBN) * ((M + kPfBM - 1) / kPfBM), steps = K / 64;
+    int ks = 1;
+    if (N % 4)
+        return 1;
+    while (ks < 16 && tiles * ks * 4 < 3 * kGemmSplitCus && steps % (ks * 4) == 0 && steps / (ks * 2) >= 16)
+        ks *= 2;
+    return ks;
+}
+
+hipError_t launch_gemm_lut(int S, const GemmArgs &a, hipStream_t st)
+{
+    const dim3 grid(static_cast<unsigned>((a.N + kPfBN - 1) / kPfBN), static_cast<unsigned>((a.M + kPfBM - 1) / kPfBM),
+                    static_cast<unsigned>(a.ksplit));
+    const dim3 block(64 * kPfWaves);
+    const size_t lds = 2 * kPfTile;
+#define SBVR_PF_LAUNCH(SS)                                                                                     \
+    {                                                                                                          \
+        static bool raised_on[16] = {};                                                                        \
+        int dev_now = 0;                                                                                       \
+        if (hipGetDevice(&dev_now) != hipSuccess || dev_now < 0 || dev_now >= 16)                              \
+            dev_now = 0;                                                                                       \
+        bool &raised = raised_on[dev_now];                                                                     \
+        if (!raised) {                                                                                         \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sbvr_gemm_lut_kernel<SS>), \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+            if (e != hipSuccess)                                                                               \
+                return e;                                                                                      \
+            raised = true;                                                                                     \
+        }                                                                                                      \
+        hipLaunchKernelGGL(sbvr_gemm_lut_kernel<SS>, grid, block, lds, st, a);                                 \
+    }                                                                                                          \
+    break
+    switch (S) {
+    case 4: SBVR_PF_LAUNCH(4);
+#ifndef SBVR_FAST_BUILD
+    case 2: SBVR_PF_LAUNCH(2);
+    case 3: SBVR_PF_LAUNCH(3);
+#endif
+    default: return hipErrorInvalidConfiguration;
+    }
+#undef SBVR_PF_LAUNCH
+    return hipGetLastError();
+}
+
 int current_cus()
 {
     int dev = 0;
@@ -3085,6 +3395,10 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G)
 {
     if (mfma_path_ok(M, N, K, S, G) || lut_path_ok(M, N, K, S, G))
         return static_cast<size_t>(M) * N * sizeof(unsigned long long);
+    if (gemm_lut_path_ok(M, N, K, S, G)) {
+        const int ks = gemm_lut_ksplit(M, N, K);
+        return ks == 1 ? 0 : static_cast<size_t>(ks) * M * N * sizeof(float);
+    }
     if (gemm_path_ok(M, N, K, S, G) && !rows32_path_ok(M, N, K, S, G))
         return gemm_workspace_bytes(M, N, K);
     return 0;
@@ -3272,6 +3586,40 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         }
     }
 
+    // More than 32 rows, 2 to 4 planes, K and G multiples of 128: the prefill kernel that decodes by table look-up
+    // (SBVR_HIP_PF_LUT=2 keeps the tile kernel: a development switch)
+    if (!(flags & 1) && aligned && env_switches().pf_lut != 2 && gemm_lut_path_ok(M, N, K, S, G) && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        GemmArgs g{};
+        g.x = static_cast<const uint16_t *>(x);
+        g.bvr = bvr;
+        g.idx = coeff_idx;
+        g.cache = static_cast<const uint16_t *>(coeff_cache);
+        g.bias = static_cast<const uint16_t *>(bias);
+        g.out = static_cast<uint16_t *>(out);
+        g.M = M; g.N = N; g.K = K; g.L = L;
+        g.steps_per_group = G / kGemmBK;
+        g.idx16 = idx_bytes == 2;
+        g.ksplit = 1;
+        const int ks = gemm_lut_ksplit(M, N, K);
+        const size_t need = ks > 1 ? static_cast<size_t>(ks) * M * N * sizeof(float) : 0;
+        if (need && workspace && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+            g.ksplit = ks;
+            g.part = static_cast<float *>(workspace);
+        }
+        if (env_switches().show_plan)
+            fprintf(stderr, "sbvr_hip table look-up prefill M=%d N=%d K=%d S=%d: ksplit=%d\n", M, N, K, S, g.ksplit);
+        hipError_t e = launch_gemm_lut(S, g, st);
+        if (e == hipSuccess && g.ksplit > 1) {
+            const size_t quads = (static_cast<size_t>(M) * N + 3) / 4;
+            hipLaunchKernelGGL(sbvr_gemm_reduce_kernel, dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256), 0, st,
+                               g.part, g.bias, g.out, M, N, g.ksplit);
+            e = hipGetLastError();
+        }
+        if (e != hipSuccess)
+            return fail(SBVR_HIP_ELAUNCH, "prefill (table look-up) launch: %s", hipGetErrorString(e));
+        g_last_kernel = g.ksplit > 1 ? SBVR_HIP_KERNEL_PREFILL_SPLIT : SBVR_HIP_KERNEL_PREFILL;
+        return SBVR_HIP_OK;
+    }
     if (!(flags & 1) && aligned && gemm_path_ok(M, N, K, S, G) && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
         GemmArgs g{};
         g.x = static_cast<const uint16_t *>(x);

@@ -165,6 +165,47 @@ def test_rows32_table_look_up_kernel_repeatable_and_without_workspace(oracle):
     check(out, yd, "not split")
 
 
+@pytest.mark.parametrize("N,K,S,G,M,L,bias", [
+    (256, 128, 4, 128, 33, 16, False),          # one pair of steps, one tile
+    (1000, 2048, 2, 128, 300, 300, True),       # ragged N and M, two planes, uint16 indices, bias; K in parts
+    (260, 4096, 3, 256, 64, 256, False),        # three planes, groups of 256, two column tiles (the second 4 columns wide)
+    (768, 1024, 4, 512, 513, 256, False),       # groups of 512, three row tiles
+    (130, 256, 4, 128, 40, 8, True),            # N not a multiple of 4: never split
+    (2048, 8192, 4, 128, 256, 256, False)])     # 8 tiles: K in 16 parts through the workspace
+def test_prefill_table_look_up_kernel(oracle, N, K, S, G, M, L, bias):
+    """More than 32 rows, 2 to 4 planes, K and G multiples of 128: the prefill kernel that decodes by table look-up
+    in registers (256 x 256 tiles), split along K or not as the shape asks."""
+    from sbvr import hip
+    split = hip._load().sbvr_hip_linear_f16_workspace(M, N, K, S, G) > 0
+    run_case(oracle, N, K, S, G, M, L, seed=N + K + M, bias=bias, expect=PREFILL_SPLIT if split else PREFILL)
+
+
+def test_prefill_kernels_agree(oracle):
+    """The same product through the entry point without a workspace (table look-up kernel, not split) and with one
+    (split): equal up to the order of the fp32 additions."""
+    import ctypes
+    import sbvr
+    from sbvr import hip, synth
+    dev = torch.device("cuda:0")
+    N, K, S, G, M, L = 1024, 4096, 4, 128, 200, 256
+    bvr, idx, cache = (t.to(dev) for t in synth.random_encoding(N, K, S, G, L, seed=71))
+    x = torch.randn((M, K), generator=torch.Generator().manual_seed(72)).to(torch.float16).to(dev)
+    split = sbvr._sbvr_linear_f16(x, bvr, idx, cache, None, bvr_len=G)
+    assert hip.last_kernel() == PREFILL_SPLIT
+    out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    vp = ctypes.c_void_p
+    rc = hip._load().sbvr_hip_linear_f16_noalloc(vp(x.data_ptr()), vp(bvr.data_ptr()), vp(idx.data_ptr()), 1, vp(cache.data_ptr()),
+                                                 None, vp(out.data_ptr()), M, N, K, S, G, L, 0,
+                                                 vp(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0 and hip.last_kernel() == PREFILL
+    torch.cuda.synchronize()
+    rms = split.float().pow(2).mean().sqrt()
+    assert ((split.float() - out.float()).abs() / torch.maximum(split.float().abs(), rms)).max().item() < 2e-3
+    _, yd = oracle.C.linear_f16(x.cpu().numpy(), bvr.cpu().numpy(), idx.cpu().numpy(), cache.cpu().numpy(), G)
+    check(out, yd, "not split")
+    check(split, yd, "split")
+
+
 def test_matches_decode_path_rows():
     """The same rows through the decode path (16 at a time) and the prefill path."""
     import sbvr
