@@ -2080,6 +2080,98 @@ constexpr int kLutWaves = 8;
 // 5..8 rows and 17.9-20.9 us at 9..16 rows for the decode kernels (13.6-16.0 with 2 planes, 19.6-22.5 with 3).
 constexpr int kLutMinRows = 9;
 
+// ---- decode by table look-up, shared by sbvr_gemm_rows32_lut_kernel and sbvr_gemm_lut_kernel (2, 3 or 4 planes)
+template <int S>
+struct LutTables {
+    static constexpr int TW = S == 4 ? 4 : (S == 3 ? 2 : 1);       // dwords of a byte table
+    uint32_t lo[TW], hi[TW];       // low and high bytes of the subset sums 0..3, 4..7, ...
+};
+
+// The 2^S subset sums of a coefficient line (sequential fp16 additions in plane order: bit for bit the weights of the
+// arithmetic decode), entries (2i, 2i + 1) as packed pairs, then as byte tables.
+template <int S>
+__device__ __forceinline__ void lut_build_tables(const uint32_t (&c)[(S + 1) / 2], LutTables<S> &t)
+{
+    v2h cc[S];
+#pragma unroll
+    for (int q = 0; q < S; ++q) {
+        const uint32_t bits = q & 1 ? c[q / 2] >> 16 : c[q / 2] & 0xffffu;
+        cc[q] = as_v2h(bits | (bits << 16));
+    }
+    v2h e[1 << (S - 1)];
+    e[0] = as_v2h((c[0] & 0xffffu) << 16);                // entries 0, 1: nothing, c0
+    e[1] = e[0] + cc[1];                                   // 2, 3
+    if constexpr (S >= 3) {
+        e[2] = e[0] + cc[2];                               // 4, 5
+        e[3] = e[1] + cc[2];                               // 6, 7
+    }
+    if constexpr (S == 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            e[4 + i] = e[i] + cc[3];                       // 8..15: the last plane is added last
+    }
+#pragma unroll
+    for (int i = 0; i < LutTables<S>::TW; ++i) {
+        const uint32_t e0 = __builtin_bit_cast(uint32_t, e[2 * i]), e1 = __builtin_bit_cast(uint32_t, e[2 * i + 1]);
+        t.lo[i] = __builtin_amdgcn_perm(e1, e0, 0x06040200u);
+        t.hi[i] = __builtin_amdgcn_perm(e1, e0, 0x07050301u);
+    }
+}
+
+// Nibble words of one word of K: nibble n of Q[p] = selector (one bit per plane) of element p + 4n.
+template <int S>
+__device__ __forceinline__ void lut_nibble_words(const uint32_t (&w)[S], uint32_t (&Q)[4])
+{
+    auto rotr = [](uint32_t v, int r) __attribute__((always_inline)) -> uint32_t {
+        return (r & 31) == 0 ? v : __builtin_amdgcn_alignbit(v, v, r & 31);
+    };
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        uint32_t v = rotr(w[0], p) & 0x11111111u;
+        v = (rotr(w[1], p - 1) & 0x22222222u) | v;
+        if constexpr (S >= 3)
+            v = (rotr(w[2], p - 2) & 0x44444444u) | v;
+        if constexpr (S == 4)
+            v = (rotr(w[3], p - 3) & 0x88888888u) | v;
+        Q[p] = v;
+    }
+}
+
+// The weights of elements p, p + 8 (w01) and p + 16, p + 24 (w23) of the word, p = 0..7, as packed fp16 pairs.
+template <int S>
+__device__ __forceinline__ void lut_look_up(const LutTables<S> &t, const uint32_t (&Q)[4], int p, uint32_t &w01, uint32_t &w23)
+{
+    const uint32_t qs = p < 4 ? Q[p & 3] : Q[p & 3] >> 4;
+    const uint32_t sel = qs & (S == 2 ? 0x03030303u : 0x07070707u);
+    uint32_t lo, hi;
+    if constexpr (S == 2) {
+        lo = __builtin_amdgcn_perm(t.lo[0], t.lo[0], sel);
+        hi = __builtin_amdgcn_perm(t.hi[0], t.hi[0], sel);
+    } else {
+        lo = __builtin_amdgcn_perm(t.lo[1], t.lo[0], sel);
+        hi = __builtin_amdgcn_perm(t.hi[1], t.hi[0], sel);
+    }
+    if constexpr (S == 4) {
+        // bytes of ones where selector bit 3 is set: a look-up in the two-entry table {0x00, 0xff}
+        const uint32_t upper = __builtin_amdgcn_perm(0x0000ff00u, 0x0000ff00u, (qs >> 3) & 0x01010101u);
+        const uint32_t lo_u = __builtin_amdgcn_perm(t.lo[3], t.lo[2], sel), hi_u = __builtin_amdgcn_perm(t.hi[3], t.hi[2], sel);
+        lo = (lo_u & upper) | (lo & ~upper);
+        hi = (hi_u & upper) | (hi & ~upper);
+    }
+    w01 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
+    w23 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
+}
+
+// The B operand of MFMA q = 0..3 of the word: elements 2q, 2q+8, 2q+16, 2q+24, 2q+1, 2q+9, 2q+17, 2q+25.
+template <int S>
+__device__ __forceinline__ v4u lut_operand(const LutTables<S> &t, const uint32_t (&Q)[4], int q)
+{
+    uint32_t b0, b1, b2, b3;
+    lut_look_up<S>(t, Q, 2 * q, b0, b1);
+    lut_look_up<S>(t, Q, 2 * q + 1, b2, b3);
+    return v4u{b0, b1, b2, b3};
+}
+
 // kHalfRows: up to 16 batch rows (the activation loads of rows 16..31 are left out); kShare: groups of a multiple
 // of 128 elements, so the two steps of a loop iteration (an even word pair and the next) share a coefficient line:
 // one index load, one gather and one table per two steps.
@@ -2094,7 +2186,6 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
     constexpr int kXRow = 144;
     __shared__ __align__(16) unsigned char xs[kLutWaves][32 * kXRow];
     constexpr int CW = (S + 1) / 2;
-    constexpr int TW = S == 4 ? 4 : (S == 3 ? 2 : 1);       // dwords of a byte table
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -2153,37 +2244,8 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
     for (int r = 0; r < 16; ++r)
         acc[r] = 0.f;
 
-    auto rotr = [](uint32_t v, int r) __attribute__((always_inline)) -> uint32_t {
-        return (r & 31) == 0 ? v : __builtin_amdgcn_alignbit(v, v, r & 31);
-    };
-    uint32_t tlo[TW], thi[TW];
-    // ---- the group's subset sums, entries (2i, 2i + 1) as packed pairs, then as byte tables
-    auto build_table = [&](const uint32_t (&c)[CW]) __attribute__((always_inline)) {
-        v2h cc[S];
-#pragma unroll
-        for (int q = 0; q < S; ++q) {
-            const uint32_t bits = q & 1 ? c[q / 2] >> 16 : c[q / 2] & 0xffffu;
-            cc[q] = as_v2h(bits | (bits << 16));
-        }
-        v2h e[1 << (S - 1)];
-        e[0] = as_v2h((c[0] & 0xffffu) << 16);                // entries 0, 1: nothing, c0
-        e[1] = e[0] + cc[1];                                   // 2, 3
-        if constexpr (S >= 3) {
-            e[2] = e[0] + cc[2];                               // 4, 5
-            e[3] = e[1] + cc[2];                               // 6, 7
-        }
-        if constexpr (S == 4) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                e[4 + i] = e[i] + cc[3];                       // 8..15: the last plane is added last
-        }
-#pragma unroll
-        for (int i = 0; i < TW; ++i) {
-            const uint32_t e0 = __builtin_bit_cast(uint32_t, e[2 * i]), e1 = __builtin_bit_cast(uint32_t, e[2 * i + 1]);
-            tlo[i] = __builtin_amdgcn_perm(e1, e0, 0x06040200u);
-            thi[i] = __builtin_amdgcn_perm(e1, e0, 0x07050301u);
-        }
-    };
+    LutTables<S> tables;
+    auto build_table = [&](const uint32_t (&c)[CW]) __attribute__((always_inline)) { lut_build_tables<S>(c, tables); };
     auto compute = [&](const Step &st) __attribute__((always_inline)) {
         // ---- activations: rows as loaded -> LDS -> a row per lane (the LDS serves a wave's accesses in order)
 #pragma unroll
@@ -2195,46 +2257,11 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
         for (int i = 0; i < 4; ++i)
             xl[i] = *reinterpret_cast<const v4u *>(xr + 16 * i);
         __builtin_amdgcn_wave_barrier();
-        // ---- nibble words: nibble n of Q[p] = selector of element p + 4n
         uint32_t Q[4];
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            uint32_t v = rotr(st.w[0], p) & 0x11111111u;
-            v = (rotr(st.w[1], p - 1) & 0x22222222u) | v;
-            if constexpr (S >= 3)
-                v = (rotr(st.w[2], p - 2) & 0x44444444u) | v;
-            if constexpr (S == 4)
-                v = (rotr(st.w[3], p - 3) & 0x88888888u) | v;
-            Q[p] = v;
-        }
-        // the weights of elements p, p + 8 (first result) and p + 16, p + 24 (second) as packed fp16 pairs
-        auto look_up = [&](int p, uint32_t &w01, uint32_t &w23) __attribute__((always_inline)) {
-            const uint32_t qs = p < 4 ? Q[p & 3] : Q[p & 3] >> 4;
-            const uint32_t sel = qs & (S == 2 ? 0x03030303u : 0x07070707u);
-            uint32_t lo, hi;
-            if constexpr (S == 2) {
-                lo = __builtin_amdgcn_perm(tlo[0], tlo[0], sel);
-                hi = __builtin_amdgcn_perm(thi[0], thi[0], sel);
-            } else {
-                lo = __builtin_amdgcn_perm(tlo[1], tlo[0], sel);
-                hi = __builtin_amdgcn_perm(thi[1], thi[0], sel);
-            }
-            if constexpr (S == 4) {
-                // bytes of ones where selector bit 3 is set: a look-up in the two-entry table {0x00, 0xff}
-                const uint32_t upper = __builtin_amdgcn_perm(0x0000ff00u, 0x0000ff00u, (qs >> 3) & 0x01010101u);
-                const uint32_t lo_u = __builtin_amdgcn_perm(tlo[3], tlo[2], sel), hi_u = __builtin_amdgcn_perm(thi[3], thi[2], sel);
-                lo = (lo_u & upper) | (lo & ~upper);
-                hi = (hi_u & upper) | (hi & ~upper);
-            }
-            w01 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
-            w23 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
-        };
+        lut_nibble_words<S>(st.w, Q);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            uint32_t b0, b1, b2, b3;
-            look_up(2 * q, b0, b1);
-            look_up(2 * q + 1, b2, b3);
-            const v4u bw = {b0, b1, b2, b3};
+            const v4u bw = lut_operand<S>(tables, Q, q);
             v4u aw;
             // dword i of the lane's 64 bytes of activations holds elements 2i, 2i + 1
             const uint32_t d0 = xl[0][q], d1 = xl[1][q], d2 = xl[2][q], d3 = xl[3][q];
@@ -2452,7 +2479,6 @@ sbvr_gemm_lut_kernel(const GemmArgs a)
     static_assert(S >= 2 && S <= 4, "tables of 4, 8 or 16 entries");
     extern __shared__ __align__(16) unsigned char psm[];
     constexpr int CW = (S + 1) / 2;
-    constexpr int TW = S == 4 ? 4 : (S == 3 ? 2 : 1);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -2509,33 +2535,8 @@ sbvr_gemm_lut_kernel(const GemmArgs a)
         }
     };
 
-    uint32_t tlo[TW], thi[TW];
-    auto build_table = [&](const uint32_t (&c)[CW]) __attribute__((always_inline)) {
-        v2h cc[S];
-#pragma unroll
-        for (int q = 0; q < S; ++q) {
-            const uint32_t bits = q & 1 ? c[q / 2] >> 16 : c[q / 2] & 0xffffu;
-            cc[q] = as_v2h(bits | (bits << 16));
-        }
-        v2h e[1 << (S - 1)];
-        e[0] = as_v2h((c[0] & 0xffffu) << 16);
-        e[1] = e[0] + cc[1];
-        if constexpr (S >= 3) {
-            e[2] = e[0] + cc[2];
-            e[3] = e[1] + cc[2];
-        }
-        if constexpr (S == 4) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                e[4 + i] = e[i] + cc[3];
-        }
-#pragma unroll
-        for (int i = 0; i < TW; ++i) {
-            const uint32_t e0 = __builtin_bit_cast(uint32_t, e[2 * i]), e1 = __builtin_bit_cast(uint32_t, e[2 * i + 1]);
-            tlo[i] = __builtin_amdgcn_perm(e1, e0, 0x06040200u);
-            thi[i] = __builtin_amdgcn_perm(e1, e0, 0x07050301u);
-        }
-    };
+    LutTables<S> tables;
+    auto build_table = [&](const uint32_t (&c)[CW]) __attribute__((always_inline)) { lut_build_tables<S>(c, tables); };
 
     v16f acc[8];
 #pragma unroll
@@ -2544,47 +2545,10 @@ sbvr_gemm_lut_kernel(const GemmArgs a)
         for (int r = 0; r < 16; ++r)
             acc[rb][r] = 0.f;
 
-    auto rotr = [](uint32_t v, int r) __attribute__((always_inline)) -> uint32_t {
-        return (r & 31) == 0 ? v : __builtin_amdgcn_alignbit(v, v, r & 31);
-    };
     auto compute = [&](const uint32_t (&w)[S], int buf) __attribute__((always_inline)) {
         uint32_t Q[4];
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            uint32_t v = rotr(w[0], p) & 0x11111111u;
-            v = (rotr(w[1], p - 1) & 0x22222222u) | v;
-            if constexpr (S >= 3)
-                v = (rotr(w[2], p - 2) & 0x44444444u) | v;
-            if constexpr (S == 4)
-                v = (rotr(w[3], p - 3) & 0x88888888u) | v;
-            Q[p] = v;
-        }
-        auto look_up = [&](int p, uint32_t &w01, uint32_t &w23) __attribute__((always_inline)) {
-            const uint32_t qs = p < 4 ? Q[p & 3] : Q[p & 3] >> 4;
-            const uint32_t sel = qs & (S == 2 ? 0x03030303u : 0x07070707u);
-            uint32_t lo, hi;
-            if constexpr (S == 2) {
-                lo = __builtin_amdgcn_perm(tlo[0], tlo[0], sel);
-                hi = __builtin_amdgcn_perm(thi[0], thi[0], sel);
-            } else {
-                lo = __builtin_amdgcn_perm(tlo[1], tlo[0], sel);
-                hi = __builtin_amdgcn_perm(thi[1], thi[0], sel);
-            }
-            if constexpr (S == 4) {
-                const uint32_t upper = __builtin_amdgcn_perm(0x0000ff00u, 0x0000ff00u, (qs >> 3) & 0x01010101u);
-                const uint32_t lo_u = __builtin_amdgcn_perm(tlo[3], tlo[2], sel), hi_u = __builtin_amdgcn_perm(thi[3], thi[2], sel);
-                lo = (lo_u & upper) | (lo & ~upper);
-                hi = (hi_u & upper) | (hi & ~upper);
-            }
-            w01 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
-            w23 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
-        };
-        auto operand = [&](int q) __attribute__((always_inline)) -> v4u {
-            uint32_t b0, b1, b2, b3;
-            look_up(2 * q, b0, b1);
-            look_up(2 * q + 1, b2, b3);
-            return v4u{b0, b1, b2, b3};
-        };
+        lut_nibble_words<S>(w, Q);
+        auto operand = [&](int q) __attribute__((always_inline)) -> v4u { return lut_operand<S>(tables, Q, q); };
         // MFMA q of all 8 row blocks in a row (8 different accumulators), its 8 activation operands read while
         // MFMA q - 1 runs, and the look-ups of operand q + 1 in the shadow of the matrix pipe
         const unsigned char *xt = xrd + buf * kPfTile;
