@@ -311,14 +311,26 @@ def prefill_leg():
     rows = []
     for n, k in ((28672, 8192), (8192, 28672)):
         w = tuple(t.to(dev) for t in synth.random_encoding(n, k, NUM_SUMS, GROUP, LINES, seed=1))
+        dense = (torch.randn((n, k), generator=torch.Generator().manual_seed(5)) * 0.02).to(torch.float16).to(dev)
         for m in (256, 512, 1024, 2048):
             x = torch.randn((m, k), generator=torch.Generator().manual_seed(6)).to(torch.float16).to(dev)
             out = torch.empty((m, n), dtype=torch.float16, device=dev)
             t = _graph_time(lambda i: hip._sbvr_linear_f16(x, *w, None, GROUP, out=out), 5)
             flops = 2.0 * m * n * k
+            # for scale: the library's GEMM on ready-made dense fp16 weights of the same shape (nothing to decode)
+            for _ in range(2):
+                torch.matmul(x, dense.t(), out=out)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(5):
+                torch.matmul(x, dense.t(), out=out)
+            e1.record()
+            torch.cuda.synchronize()
+            t_dense = e0.elapsed_time(e1) * 1e-3 / 5
             rows.append({"N": n, "K": k, "M": m, "us": round(t * 1e6, 1), "TFLOPs": round(flops / t / 1e12, 1),
-                         "frac_of_fp16_mfma_peak": round(flops / t / 1e12 / 2500.0, 4)})
-        del w
+                         "frac_of_fp16_mfma_peak": round(flops / t / 1e12 / 2500.0, 4),
+                         "dense_fp16_library_gemm_us": round(t_dense * 1e6, 1)})
+        del w, dense
         torch.cuda.empty_cache()
     return rows
 
