@@ -133,18 +133,29 @@ def gpu_leg(steps, warmup, floor=False):
     return wall_ms, timing, launcher, torch.cuda.get_device_name(0)
 
 
-def decode_leg(prompt_tokens=128, new_tokens=128):
-    """Random-init Llama-3-8B-shaped decoder with SBVR linears (sbvr/decoder.py):
-    a 128-token uniform-random prompt, then 128 greedy tokens at batch 1, one
-    HIP-graph replay per token; the figure covers the new tokens only."""
+def decode_workload(prompt_tokens=128, new_tokens=128):
+    """The decoder and the prompt of the "8B decode tokens/s" figure (BASELINE.json configs[3]): 32 layers at the
+    Llama-3-8B widths, random init, seeded synthetic encodings, a 128-token uniform-random prompt.  Also what
+    tests/test_gpu_config4.py checks against the oracle."""
     import torch
     from sbvr.decoder import LlamaShape, SbvrLlamaDecoder
 
     shape = LlamaShape()
     dec = SbvrLlamaDecoder(shape, "cuda:0", num_sums=NUM_SUMS, bvr_len=GROUP, lines=LINES,
                            max_seq=prompt_tokens + new_tokens)
-    dec.capture()
     prompt = torch.randint(0, shape.vocab, (prompt_tokens,), generator=torch.Generator().manual_seed(0))
+    return dec, prompt
+
+
+def decode_leg(prompt_tokens=128, new_tokens=128):
+    """Random-init Llama-3-8B-shaped decoder with SBVR linears (sbvr/decoder.py):
+    a 128-token uniform-random prompt, then 128 greedy tokens at batch 1, one
+    HIP-graph replay per token; the figure covers the new tokens only."""
+    import torch
+
+    dec, prompt = decode_workload(prompt_tokens, new_tokens)
+    shape = dec.shape
+    dec.capture()
     best = None
     for _ in range(2):
         tokens, seconds = dec.generate(prompt, new_tokens)
@@ -231,6 +242,69 @@ def _graph_time(fn, iters, stream=None):
             t = e0.elapsed_time(e1) * 1e-3 / iters
             best = t if best is None else min(best, t)
     return best
+
+
+def read_floor_leg(quick=False):
+    """What the memory system hands to a launch that only reads, whatever grid the decode kernel uses
+    (sbvr_hip_read_floor): the 28 672 KiB of plane words of the gate shape, one request of 1 KiB per wave
+    instruction, over workgroups per CU in {1, 2, 4} x waves in {4, 8, 16} x requests in flight per wave, as one
+    contiguous band (pattern 0), a contiguous piece per wave (1) and in the decode kernel's own 896-byte windows
+    of 229 376-byte rows (2); plus one stream of 1 GiB.  The buffers rotate through the same 16 weight copies as
+    the timed GEMV (beyond the 256 MB memory-side cache).  quick: the few shapes the default line reports."""
+    import torch
+    from sbvr import hip
+    dev = torch.device("cuda:0")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    plane_bytes = N_OUT * K_IN * NUM_SUMS // 8
+    bufs = [torch.randint(-2 ** 31, 2 ** 31, (plane_bytes // 4,), dtype=torch.int32, device=dev) for _ in range(COPIES)]
+    rows = []
+
+    def one(wgs_per_cu, waves, ahead, pattern):
+        wgs = cus * wgs_per_cu
+        units = plane_bytes // 1024
+        per_wave = units // (wgs * waves)
+        if pattern == 2:
+            # the gate launch's own geometry: one window of 56 columns x 16 bytes per workgroup
+            wgs, win, row = 256, 56 * NUM_SUMS * 4, N_OUT * NUM_SUMS * 4
+            per_wave = (K_IN // 128 // waves) * 4            # 4 tiles of 256 bytes (the last one half used) per sub-group
+            if K_IN // 128 % waves or per_wave % ahead:
+                return
+            nbytes = per_wave * wgs * waves * 1024
+            t = _graph_time(lambda i: hip.read_floor(bufs[i % COPIES], nbytes, wgs, waves, ahead, 2, row, win), 64)
+            moved = plane_bytes                                # (bytes of the buffer actually touched)
+        else:
+            if per_wave == 0 or per_wave % ahead:
+                return
+            nbytes = per_wave * wgs * waves * 1024
+            t = _graph_time(lambda i: hip.read_floor(bufs[i % COPIES], nbytes, wgs, waves, ahead, pattern), 64)
+            moved = nbytes
+        rows.append({"pattern": pattern, "workgroups_per_cu": wgs_per_cu if pattern != 2 else 1, "waves": waves, "in_flight": ahead,
+                     "KiB_per_wave": per_wave, "bytes": moved, "us": round(t * 1e6, 3),
+                     "GBps": round(moved / t / 1e9, 1), "frac_of_hbm_peak": round(moved / t / 1e9 / HBM_PEAK_GBS, 4)})
+
+    if quick:
+        grid = [(1, 16, 7, 0), (2, 8, 7, 0), (1, 8, 14, 0), (4, 4, 7, 0), (1, 16, 4, 2), (1, 16, 8, 2)]
+    else:
+        grid = [(w, v, a, p) for p in (0, 1) for w in (1, 2, 4) for v in (4, 8, 16) for a in (1, 2, 4, 7, 14)]
+        grid += [(1, v, a, 2) for v in (8, 16) for a in (1, 2, 4, 8, 16)]
+    for w, v, a, p in grid:
+        one(w, v, a, p)
+    del bufs
+    torch.cuda.empty_cache()
+    best = max(rows, key=lambda r: r["GBps"]) if rows else None
+    out = {"rows": rows, "best": best}
+    if not quick:
+        big = torch.randint(-2 ** 31, 2 ** 31, ((1 << 30) // 4,), dtype=torch.int32, device=dev)
+        big2 = torch.randint(-2 ** 31, 2 ** 31, ((1 << 30) // 4,), dtype=torch.int32, device=dev)
+        pair = (big, big2)
+        streams = []
+        for wgs_per_cu, waves, ahead in ((4, 16, 4), (8, 8, 8), (4, 16, 16), (16, 4, 16)):
+            wgs = cus * wgs_per_cu
+            t = _graph_time(lambda i: hip.read_floor(pair[i % 2], 1 << 30, wgs, waves, ahead, 0), 8)
+            streams.append({"workgroups_per_cu": wgs_per_cu, "waves": waves, "in_flight": ahead, "us": round(t * 1e6, 1),
+                            "GBps": round((1 << 30) / t / 1e9, 1), "frac_of_hbm_peak": round((1 << 30) / t / 1e9 / HBM_PEAK_GBS, 4)})
+        out["one_GiB_stream"] = streams
+    return out
 
 
 def sweep_leg():
@@ -441,6 +515,9 @@ def main():
     ap.add_argument("--stream-floor", action="store_true",
                     help="run only the launch that makes the gate GEMV's memory requests and nothing else "
                          "(sbvr_hip_linear_f16_stream_floor) and print its time beside the kernel's")
+    ap.add_argument("--read-floor", action="store_true",
+                    help="run only the launches that read 28 MiB and do nothing else, over grids, depths and access "
+                         "patterns (sbvr_hip_read_floor), and print them")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size kernel that "
                          "hardware byte counters are scaled by when profiling")
@@ -456,6 +533,9 @@ def main():
         return
     if a.prefill:
         print(json.dumps({"metric": "SBVR prefill GEMM, dense-equivalent TFLOP/s", "prefill": prefill_leg()}))
+        return
+    if a.read_floor:
+        print(json.dumps({"metric": "read-only launches of the gate shape's plane words, us and GB/s", "read_floor": read_floor_leg()}))
         return
     if a.other_ops:
         print(json.dumps({"metric": "SBVR operator forms of the reference, us and GB/s of algorithmic bytes",

@@ -31,7 +31,7 @@ extern "C" {
 #define SBVR_HIP_EWORKSPACE (-4)  /* workspace missing or too small */
 
 /* ABI version of this header (major*100 + minor); 101 added the one-row linears with a fused prologue,
- * 102 sbvr_hip_linear_f16_noalloc and sbvr_hip_linear_f16_stream_floor. */
+ * 102 sbvr_hip_linear_f16_noalloc and sbvr_hip_linear_f16_stream_floor, 103 sbvr_hip_read_floor. */
 int sbvr_hip_version(void);
 
 /* Text of the last error raised on this thread ("" if none). */
@@ -46,6 +46,17 @@ const char *sbvr_hip_last_error(void);
 #define SBVR_HIP_KERNEL_PREFILL 4        /* weights decoded to fp16 tiles in LDS */
 #define SBVR_HIP_KERNEL_PREFILL_SPLIT 5  /* the same with K split across workgroups (workspace given) */
 int sbvr_hip_last_kernel(void);
+
+/* How that launch treated the weights (0 before the first):
+ *   EXACT      coefficients applied to plane sums in fp32, no per-weight rounding (decode and portable kernels);
+ *   DECODE     every weight rounded to fp16 once, as decode() of sbvr/core.py:927-949 produces it (bin_combs @
+ *              coeff, :345-366): the kernels that decode by table look-up;
+ *   PLANEWISE  every weight an fp16 sum built plane by plane, S - 1 roundings (the kernels that decode
+ *              arithmetically: 6 and 8 planes, groups of 32 or 64 elements). */
+#define SBVR_HIP_ROUNDING_EXACT 1
+#define SBVR_HIP_ROUNDING_DECODE 2
+#define SBVR_HIP_ROUNDING_PLANEWISE 3
+int sbvr_hip_last_rounding(void);
 
 /* Checks that `device` is a gfx950 part and caches its properties.
  * Replaces sbvr_cuda_init, sbvr/kernels/sbvr_ops.cpp:122-150. */
@@ -130,9 +141,14 @@ int sbvr_hip_linear_f16(const void *x, const uint32_t *bvr, const void *coeff_id
  * that forbid hipMalloc).  It has no counterpart in the reference.  Same
  * arguments and results as sbvr_hip_linear_f16 without the workspace pair: the
  * split-K accumulators of the decode and 32-row kernels live in a 4 MiB array
- * inside the library (one copy per GPU, held until the process ends), so up to
- * 32 rows need M * N <= 524288 (SBVR_HIP_EWORKSPACE beyond that); with more rows
- * the prefill kernel runs without its optional workspace, i.e. not split along K.
+ * inside the library (one copy per GPU, held until the process ends), which
+ * holds M * N <= 524288 of them.  The one limit, up to 32 rows: a launch that
+ * splits K across workgroups and has more outputs than that runs unsplit where
+ * its kernel can (the table look-up kernel of 9 to 32 rows) and is refused
+ * with SBVR_HIP_EWORKSPACE where it cannot (the decode kernels, up to 8 rows);
+ * launches that do not split K never touch the array and have no limit.  With
+ * more than 32 rows the prefill kernel runs without its optional workspace,
+ * i.e. not split along K.
  * The call allocates and frees nothing.  Calls that overlap in time on one GPU
  * share the array and race: serialise them (one stream, or events).
  */
@@ -184,6 +200,35 @@ int sbvr_hip_linear_f16_stream_floor(const uint32_t *bvr, const void *coeff_idx,
                                      void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: a launch that only reads
+ * `bytes` of buf (a buffer of buf_bytes), whatever grid the linear would use:
+ * `workgroups` x `waves` waves (waves <= 16) each request bytes / 1024 /
+ * (workgroups * waves) units of 1 KiB, one 16-byte load per lane (the decode
+ * kernel's request), `ahead` of them in flight (1, 2, 3, 4, 7, 8, 14 or 16; a
+ * divisor of the units per wave), and do nothing else.  pattern 0: at any time
+ * the grid reads one contiguous band (unit i of wave w is KiB i * waves_total
+ * + w); 1: every wave walks its own contiguous piece; 2: the decode kernel's
+ * own pattern over rows of row_bytes (one 32-bit word of K for all columns)
+ * with win_bytes of every row per workgroup and 256 bytes of four consecutive
+ * rows per unit.  sink: 256 bytes of device memory, never written.  bench.py
+ * --read-floor times it over weight copies that rotate through more than the
+ * 256 MB memory-side cache.
+ */
+int sbvr_hip_read_floor(const void *buf, size_t buf_bytes, size_t bytes, int workgroups, int waves, int ahead,
+                        int pattern, int row_bytes, int win_bytes, void *sink, void *stream);
+
+/*
+ * Query, no counterpart in the reference and no device needed: the launch shape
+ * the decode kernels would get for M <= 16 rows of this shape on a device of
+ * `cus` compute units.  plan[0..7] = {kind, column tiles per wave, sub-groups
+ * of 128 per wave, row tiles, waves per workgroup, column windows, parts of K
+ * across workgroups, the most waves the kernel instance may be launched with};
+ * kind 1: sbvr_gemv_mfma_kernel, 2: sbvr_gemv_batch_kernel, 0 (all zero): the
+ * decode kernels do not cover the shape.
+ */
+int sbvr_hip_decode_plan(int M, int N, int K, int S, int G, int cus, int *plan);
+
+/*
  * fp16 activations against a weight encoded with trans=True (groups along N):
  *   r_bvr (N/32, K, S) uint32, r_coeff_idx (N/G, K), r_coeff_cache (L, S) fp16
  *   out[m,n] = f16( bias[n] + sum_k x[m,k] * sum_j c[idx[n/G,k], j] * bit_j )
@@ -199,7 +244,8 @@ int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_co
  * The same product with room for a split of K across workgroups: a workspace of
  * sbvr_hip_row_deq_mm_T_workspace(M, N) bytes (M*N 64-bit accumulators, zero-filled once, 8-byte
  * aligned, left zero by every call; it may be the workspace of sbvr_hip_linear_f16, not used by
- * two calls at once).  With 4 planes, K a multiple of 128 and groups of 64 columns and more the
+ * two calls at once; 0 bytes for a call whose column workgroups already fill the device: it is
+ * never split, e.g. any prefill-sized M).  With 4 planes, K a multiple of 128 and groups of 64 columns and more the
  * plane sums run on the matrix cores, and where the columns alone would leave CUs idle (N = 4096
  * on an MI355X) the parts of K are summed through the accumulators, in fixed point, so the result
  * does not depend on their order.  workspace NULL: as sbvr_hip_row_deq_mm_T.  The reference's

@@ -65,6 +65,7 @@ typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
 thread_local char g_err[256] = "";
 thread_local int g_last_kernel = 0;       // SBVR_HIP_KERNEL_* of the last linear launched from this thread
+thread_local int g_last_rounding = 0;     // SBVR_HIP_ROUNDING_* of that launch
 
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int fail(int code, const char *fmt, ...)
@@ -81,6 +82,7 @@ struct DevInfo {
     int cus = 256;
 };
 DevInfo g_dev[16];
+std::mutex g_dev_lock;           // guards g_dev[] and the scratch addresses: first use may come from several threads
 
 // ------------------------------------------------------------------ helpers
 
@@ -1087,11 +1089,21 @@ struct GemvPlan {
     int wstride;
 };
 
-// Development switches, read from the environment once per process.
+// Development switches.  A library built with -DSBVR_DEV_SWITCHES reads them from the environment once per
+// process (SBVR_HIP_CT, _SP, _WAVES, _WSTRIDE, _SHOW_PLAN, _POPC_Q, _ROWDEQ_LANES, _LUT_ROWS, _PF_LUT); the
+// library as shipped does not look at the environment: launch shapes and the choice of kernel (and with it the
+// rounding) depend on the arguments of a call alone.
 struct EnvSwitches {
     int ct, sp, waves, wstride, show_plan, popc_q, rowdeq_lanes, lut_rows, pf_lut;
 };
 
+#ifndef SBVR_DEV_SWITCHES
+const EnvSwitches &env_switches()
+{
+    static const EnvSwitches none{};
+    return none;
+}
+#else
 const EnvSwitches &env_switches()
 {
     static const EnvSwitches e = [] {
@@ -1104,6 +1116,7 @@ const EnvSwitches &env_switches()
     }();
     return e;
 }
+#endif
 
 // (CT, SP) pairs that have a kernel instance; see the dispatch below.
 constexpr int kShapes[][2] = {{1, 1}, {1, 2}, {1, 4}, {1, 7}, {2, 1}, {2, 2}, {2, 4}, {2, 7}, {4, 1}, {4, 2}, {4, 4}, {7, 2}};
@@ -1150,7 +1163,7 @@ GemvPlan plan_gemv_uncached(int M, int N, int K, int S, int cus, int min_waves)
     // workgroups with four sub-groups a wave measured 14.1-14.7 us against 16.0 for 16 waves with two at
     // 4096 -> 28672, and only that large a matrix gains from taking all of K into the workgroup)
     const bool norm = min_waves > 1;
-    const int wg_waves = norm ? 8 : kMaxWaves;
+    const int wg_waves = norm ? 8 : std::min(kMaxWaves, gemv_max_waves(MT, 0));      // (never above the kernel's launch bound)
     if (best.CT == 0 && eCT <= 0 && nsub % wg_waves == 0 && wg_waves >= min_waves && N >= (norm ? 64 : 16) * cus) {
         const int SP = nsub / wg_waves;
         // windows of wstride columns, r workgroups per CU; without the prologue one workgroup per CU takes up
@@ -1256,6 +1269,7 @@ hipError_t launch_gemv_inst(const GemvArgs &a, const GemvPlan &p, hipStream_t st
     const dim3 grid(static_cast<unsigned>(p.n_wgs), static_cast<unsigned>(p.ksplit)), block(64 * p.waves);
     if (p.lds > 65536) {        // (the wide shapes' partial results) above what a kernel gets without asking
         static bool raised_on[16] = {};
+        std::lock_guard<std::mutex> guard(g_dev_lock);
         int dev_now = 0;
         if (hipGetDevice(&dev_now) != hipSuccess || dev_now < 0 || dev_now >= 16)
             dev_now = 0;
@@ -1420,6 +1434,7 @@ hipError_t launch_batch_inst(const GemvArgs &a, const BatchPlan &p, hipStream_t 
     const dim3 grid(static_cast<unsigned>(p.n_wgs), static_cast<unsigned>(p.ksplit)), block(64 * p.waves);
     if (p.lds > 65536) {        // above what a kernel gets without asking
         static bool raised_on[16] = {};
+        std::lock_guard<std::mutex> guard(g_dev_lock);
         int dev_now = 0;
         if (hipGetDevice(&dev_now) != hipSuccess || dev_now < 0 || dev_now >= 16)
             dev_now = 0;
@@ -2061,7 +2076,7 @@ hipError_t launch_rows32(int S, RowsArgs a, hipStream_t st)
 // The same contraction as sbvr_gemm_rows32_kernel (batch rows = the 32 rows of v_mfma_f32_32x32x16_f16, 32
 // columns of decoded fp16 weights as B), with a cheaper decode for 2, 3 and 4 planes.  A weight of a group is
 // one of the 2^S subset sums of the group's coefficient line; the lane builds those once per group
-// (sequential fp16 additions in plane order, the sums the arithmetic decode produces bit for bit) and keeps
+// (each the fp32 sum rounded to fp16 once, as the reference's decode() rounds a weight) and keeps
 // them as byte tables: the low bytes of entries 0..3, 4..7, ... and the high bytes likewise.  A lane owns a
 // whole word of K per step (half h of the wave takes word 2i + h of the word pair i).  Its plane words are
 // merged into four "nibble words" Q_p, p = 0..3: nibble n of Q_p is the S-bit selector of element p + 4n, at
@@ -2087,28 +2102,32 @@ struct LutTables {
     uint32_t lo[TW], hi[TW];       // low and high bytes of the subset sums 0..3, 4..7, ...
 };
 
-// The 2^S subset sums of a coefficient line (sequential fp16 additions in plane order: bit for bit the weights of the
-// arithmetic decode), entries (2i, 2i + 1) as packed pairs, then as byte tables.
+// The 2^S subset sums of a coefficient line, entries (2i, 2i + 1) as packed pairs, then as byte tables.  Entry i is
+// the sum of the coefficients whose bit is set in i, added up in fp32 and rounded to fp16 once: the reference's
+// decode() takes a weight from bin_combs @ coeff (sbvr/core.py:345-366, 927-949), the exact sum rounded once.  The
+// fp32 sums are exact, and the entries therefore decode()'s weights bit for bit, whenever the exponents of a line's
+// coefficients lie within 11 of each other (every partial sum is then a multiple of the smallest coefficient's
+// last place below 2^24 of them); a line that mixes coefficients 2^12 apart and more can differ from decode() in
+// the last place of an entry that lands on a rounding tie.
 template <int S>
 __device__ __forceinline__ void lut_build_tables(const uint32_t (&c)[(S + 1) / 2], LutTables<S> &t)
 {
-    v2h cc[S];
+    float cf[S];
 #pragma unroll
-    for (int q = 0; q < S; ++q) {
-        const uint32_t bits = q & 1 ? c[q / 2] >> 16 : c[q / 2] & 0xffffu;
-        cc[q] = as_v2h(bits | (bits << 16));
-    }
+    for (int q = 0; q < S; ++q)
+        cf[q] = h2f(static_cast<uint16_t>(q & 1 ? c[q / 2] >> 16 : c[q / 2] & 0xffffu));
+    float s[1 << S];
+    s[0] = 0.f;
+#pragma unroll
+    for (int q = 0; q < S; ++q)
+#pragma unroll
+        for (int i = 0; i < (1 << q); ++i)
+            s[(1 << q) + i] = i == 0 ? cf[q] : s[i] + cf[q];
     v2h e[1 << (S - 1)];
-    e[0] = as_v2h((c[0] & 0xffffu) << 16);                // entries 0, 1: nothing, c0
-    e[1] = e[0] + cc[1];                                   // 2, 3
-    if constexpr (S >= 3) {
-        e[2] = e[0] + cc[2];                               // 4, 5
-        e[3] = e[1] + cc[2];                               // 6, 7
-    }
-    if constexpr (S == 4) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            e[4 + i] = e[i] + cc[3];                       // 8..15: the last plane is added last
+    for (int i = 0; i < (1 << (S - 1)); ++i) {
+        e[i][0] = static_cast<_Float16>(s[2 * i]);         // (one v_cvt_pk_f16_f32 per pair, round to nearest even)
+        e[i][1] = static_cast<_Float16>(s[2 * i + 1]);
     }
 #pragma unroll
     for (int i = 0; i < LutTables<S>::TW; ++i) {
@@ -2427,6 +2446,7 @@ hipError_t launch_gemm(int S, const GemmArgs &a, hipStream_t st)
 #define SBVR_GEMM_LAUNCH(SS)                                                                                   \
     {                                                                                                          \
         static bool raised_on[16] = {};                                                                        \
+        std::lock_guard<std::mutex> guard(g_dev_lock);                                                                        \
         int dev_now = 0;                                                                                       \
         if (hipGetDevice(&dev_now) != hipSuccess || dev_now < 0 || dev_now >= 16)                              \
             dev_now = 0;                                                                                       \
@@ -2674,6 +2694,7 @@ hipError_t launch_gemm_lut(int S, const GemmArgs &a, hipStream_t st)
 #define SBVR_PF_LAUNCH(SS)                                                                                     \
     {                                                                                                          \
         static bool raised_on[16] = {};                                                                        \
+        std::lock_guard<std::mutex> guard(g_dev_lock);                                                                        \
         int dev_now = 0;                                                                                       \
         if (hipGetDevice(&dev_now) != hipSuccess || dev_now < 0 || dev_now >= 16)                              \
             dev_now = 0;                                                                                       \
@@ -2705,6 +2726,7 @@ int current_cus()
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16)
         return 256;
+    std::lock_guard<std::mutex> guard(g_dev_lock);
     if (!g_dev[dev].ready) {
         hipDeviceProp_t prop;
         if (hipGetDeviceProperties(&prop, dev) == hipSuccess) {
@@ -3277,6 +3299,57 @@ bool launch_mm_T_popc_sr(int Sr, int Q, hipStream_t st, const uint32_t *l_bvr, c
 
 } // namespace
 
+// ---- measurement aid: a launch that only reads.  What the memory system of the part hands to a launch of a given
+// size, whatever grid the decode kernel happens to use: every wave requests `units` units of 1 KiB (one
+// global_load_dwordx4 per lane: the decode kernel's request) and keeps AHEAD of them in flight; nothing else.
+//   pattern 0: unit i of wave w is KiB number i * (waves of the grid) + w of the buffer: at any time the grid
+//              reads one contiguous band;
+//   pattern 1: unit i of wave w is KiB number w * units + i: every wave walks its own contiguous piece;
+//   pattern 2: the decode kernel's own: the buffer is rows of `row_bytes` (one word of K for all columns), a
+//              workgroup owns `win_bytes` of every row and its waves split the rows; a unit is 256 bytes of four
+//              consecutive rows (lanes past the window repeat its last 16 bytes, as the kernel's lanes do).
+namespace {
+
+template <int AHEAD>
+__global__ void __launch_bounds__(1024)
+sbvr_read_floor_kernel(const v4u *__restrict__ base, uint32_t units, int pattern, uint32_t row_bytes, uint32_t win_bytes,
+                       uint32_t *__restrict__ sink)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), waves = blockDim.x >> 6;
+    const uint32_t gw = blockIdx.x * waves + wave, total = gridDim.x * waves;
+    const uint32_t tiles = (win_bytes + 255u) / 256u;            // pattern 2: units per four rows of the window
+    auto unit_ptr = [&](uint32_t i) __attribute__((always_inline)) -> const v4u * {
+        if (pattern == 2) {
+            const uint32_t sg = wave * (units / tiles) + i / tiles, ct = i % tiles;
+            const size_t row = static_cast<size_t>(4u * sg + (lane >> 4));
+            const uint32_t in_win = min(ct * 256u + (lane & 15u) * 16u, win_bytes - 16u);
+            return reinterpret_cast<const v4u *>(reinterpret_cast<const unsigned char *>(base) + row * row_bytes +
+                                                 static_cast<size_t>(blockIdx.x) * win_bytes + in_win);
+        }
+        const size_t kib = pattern == 0 ? static_cast<size_t>(i) * total + gw : static_cast<size_t>(gw) * units + i;
+        return base + kib * 64u + lane;
+    };
+    v4u q[AHEAD], seen = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j)
+        q[j] = __builtin_nontemporal_load(unit_ptr(static_cast<uint32_t>(j)));
+    for (uint32_t i = AHEAD; i < units; i += AHEAD) {             // (units is a multiple of AHEAD: checked by the host)
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) {
+            seen ^= q[j];
+            q[j] = __builtin_nontemporal_load(unit_ptr(i + static_cast<uint32_t>(j)));
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j)
+        seen ^= q[j];
+    if ((seen.x ^ seen.y ^ seen.z ^ seen.w) == 0x9e3779b9u && units == 0x7fffffffu)      // never true: keeps the loads alive
+        sink[lane] = seen.x;
+}
+
+} // namespace
+
 // Scratch memory of sbvr_hip_linear_f16_noalloc: the split-K accumulators of the decode kernel, for callers
 // that cannot bring a workspace.  One copy per GPU the library runs on, held until the process ends; zero when
 // the module is loaded, and every launch leaves it zero (the adder that completes an accumulator resets it).
@@ -3298,6 +3371,7 @@ int scratch_on_current_device(void **out)
         return fail(SBVR_HIP_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
     if (dev < 0 || dev >= 16)
         return fail(SBVR_HIP_EUNSUPPORTED, "device %d: this library keeps scratch memory for devices 0..15", dev);
+    std::lock_guard<std::mutex> guard(g_dev_lock);
     if (!g_scratch_ptr[dev]) {
         void *ptr = nullptr;
         e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
@@ -3319,11 +3393,13 @@ extern "C" {
 void sbvr_hip_debug_set_trace(unsigned long long *p) { g_trace = p; }
 #endif
 
-int sbvr_hip_version(void) { return 102; }      // 101: the one-row linears with a fused prologue; 102: _noalloc, _stream_floor
+int sbvr_hip_version(void) { return 103; }      // 101: the one-row linears with a fused prologue; 102: _noalloc, _stream_floor; 103: _read_floor
 
 const char *sbvr_hip_last_error(void) { return g_err; }
 
 int sbvr_hip_last_kernel(void) { return g_last_kernel; }
+
+int sbvr_hip_last_rounding(void) { return g_last_rounding; }
 
 int sbvr_hip_init(int device)
 {
@@ -3340,8 +3416,11 @@ int sbvr_hip_init(int device)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(SBVR_HIP_EUNSUPPORTED, "device %d is %s; this library is built for gfx950 only",
                     device, prop.gcnArchName);
-    g_dev[device].cus = prop.multiProcessorCount;
-    g_dev[device].ready = true;
+    {
+        std::lock_guard<std::mutex> guard(g_dev_lock);
+        g_dev[device].cus = prop.multiProcessorCount;
+        g_dev[device].ready = true;
+    }
     // the scratch array's address on this device (each GPU holds its own copy at its own address)
     int before = 0;
     if (hipGetDevice(&before) != hipSuccess)
@@ -3443,6 +3522,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "rows32 (table look-up) launch: %s", hipGetErrorString(e));
         g_last_kernel = SBVR_HIP_KERNEL_ROWS32;
+        g_last_rounding = SBVR_HIP_ROUNDING_DECODE;
         return SBVR_HIP_OK;
     }
     if (pro.mode == kXPlain && !(flags & 3) && aligned && rows32_preferred(M, N, K, S, G, current_cus()) && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
@@ -3460,6 +3540,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "rows32 launch: %s", hipGetErrorString(e));
         g_last_kernel = SBVR_HIP_KERNEL_ROWS32;
+        g_last_rounding = SBVR_HIP_ROUNDING_PLANEWISE;
         return SBVR_HIP_OK;
     }
     if (pro.mode == kXPlain && !(flags & 1) && aligned && batch_path_ok(M, N, K, S, G)) {
@@ -3496,6 +3577,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
             if (e != hipSuccess)
                 return fail(SBVR_HIP_ELAUNCH, "batch launch (MT=%d CTW=%d SP=%d waves=%d ksplit=%d): %s", p.MT, p.CTW, p.SP, p.waves, p.ksplit, hipGetErrorString(e));
             g_last_kernel = SBVR_HIP_KERNEL_DECODE;
+            g_last_rounding = SBVR_HIP_ROUNDING_EXACT;
             return SBVR_HIP_OK;
         }
     }
@@ -3546,6 +3628,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "gemv launch (CT=%d SP=%d MT=%d waves=%d ksplit=%d): %s", p.CT, p.SP, p.MT, p.waves, p.ksplit, hipGetErrorString(e));
         g_last_kernel = SBVR_HIP_KERNEL_DECODE;
+        g_last_rounding = SBVR_HIP_ROUNDING_EXACT;
         return SBVR_HIP_OK;
         }
     }
@@ -3582,6 +3665,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "prefill (table look-up) launch: %s", hipGetErrorString(e));
         g_last_kernel = g.ksplit > 1 ? SBVR_HIP_KERNEL_PREFILL_SPLIT : SBVR_HIP_KERNEL_PREFILL;
+        g_last_rounding = SBVR_HIP_ROUNDING_DECODE;
         return SBVR_HIP_OK;
     }
     if (!(flags & 1) && aligned && gemm_path_ok(M, N, K, S, G) && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
@@ -3616,6 +3700,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
         if (e != hipSuccess)
             return fail(SBVR_HIP_ELAUNCH, "gemm launch: %s", hipGetErrorString(e));
         g_last_kernel = g.ksplit > 1 ? SBVR_HIP_KERNEL_PREFILL_SPLIT : SBVR_HIP_KERNEL_PREFILL;
+        g_last_rounding = SBVR_HIP_ROUNDING_PLANEWISE;
         return SBVR_HIP_OK;
     }
 
@@ -3633,6 +3718,7 @@ int linear_core(const void *x, const uint32_t *bvr, const void *coeff_idx,
     if (e != hipSuccess)
         return fail(SBVR_HIP_ELAUNCH, "portable launch: %s", hipGetErrorString(e));
     g_last_kernel = SBVR_HIP_KERNEL_PORTABLE;
+    g_last_rounding = SBVR_HIP_ROUNDING_EXACT;
     return SBVR_HIP_OK;
 }
 
@@ -3657,20 +3743,26 @@ int sbvr_hip_linear_f16_noalloc(const void *x, const uint32_t *bvr, const void *
 {
     // The accumulators of the decode and 32-row kernels come from the library's own scratch array; the prefill
     // kernel runs without its optional workspace (not split along K).  Nothing is allocated or freed on the way.
+    // A launch of up to 32 rows that splits K across workgroups takes its M * N accumulators from the scratch
+    // array; one whose accumulators would not fit gets no workspace at all: the table look-up kernel (9 to 32
+    // rows) then runs unsplit, and only a decode launch (up to 8 rows) whose shape cannot do without the split
+    // is refused.
     void *ws = nullptr;
     size_t ws_bytes = 0;
-    if (M >= 1 && N >= 1 && (mfma_path_ok(M, N, K, S, G) || lut_path_ok(M, N, K, S, G)) && !(flags & 1)) {
-        const size_t need = static_cast<size_t>(M) * N * sizeof(unsigned long long);
-        if (need > kScratchBytes)
-            return fail(SBVR_HIP_EWORKSPACE, "sbvr_hip_linear_f16_noalloc takes M * N <= %zu for up to 32 rows (M=%d N=%d); "
-                        "use sbvr_hip_linear_f16 with a workspace", kScratchBytes / sizeof(unsigned long long), M, N);
+    if (M >= 1 && N >= 1 && (mfma_path_ok(M, N, K, S, G) || lut_path_ok(M, N, K, S, G)) && !(flags & 1) &&
+        static_cast<size_t>(M) * N * sizeof(unsigned long long) <= kScratchBytes) {
         const int rc = scratch_on_current_device(&ws);
         if (rc != SBVR_HIP_OK)
             return rc;
         ws_bytes = kScratchBytes;
     }
-    return linear_core(x, bvr, coeff_idx, idx_bytes, coeff_cache, bias, out, M, N, K, S, G, L, ws, ws_bytes, flags,
-                       stream, Prologue{kXPlain, nullptr, nullptr, nullptr, 0.f});
+    const int rc = linear_core(x, bvr, coeff_idx, idx_bytes, coeff_cache, bias, out, M, N, K, S, G, L, ws, ws_bytes, flags,
+                               stream, Prologue{kXPlain, nullptr, nullptr, nullptr, 0.f});
+    if (rc == SBVR_HIP_EWORKSPACE)
+        return fail(SBVR_HIP_EWORKSPACE, "sbvr_hip_linear_f16_noalloc: this launch splits K across workgroups and its M * N = %zu "
+                    "accumulators exceed the %zu of the library's scratch array; use sbvr_hip_linear_f16 with a workspace",
+                    static_cast<size_t>(M) * N, kScratchBytes / sizeof(unsigned long long));
+    return rc;
 }
 
 int sbvr_hip_linear_f16_swiglu(const void *gate_up, const uint32_t *bvr, const void *coeff_idx,
@@ -3799,14 +3891,20 @@ int sbvr_hip_row_deq_mm_T(const void *x, const uint32_t *r_bvr, const void *r_co
     return sbvr_hip_row_deq_mm_T_ws(x, r_bvr, r_coeff_idx, idx_bytes, r_coeff_cache, bias, out, M, N, K, S, G, L, nullptr, 0, stream);
 }
 
+// (the launch splits K only while its column workgroups cover less than three quarters of the CUs: the predicate
+// of sbvr_hip_row_deq_mm_T_ws; a prefill-sized call needs nothing)
 size_t sbvr_hip_row_deq_mm_T_workspace(int M, int N)
 {
-    return M > 0 && N > 0 ? static_cast<size_t>(M) * N * sizeof(unsigned long long) : 0;
+    if (M <= 0 || N <= 0)
+        return 0;
+    const long col_wgs = static_cast<long>((N / 32 + 1) / 2) * M;
+    return col_wgs * 2 < 3L * current_cus() / 4 ? static_cast<size_t>(M) * N * sizeof(unsigned long long) : 0;
 }
 
+// (only one left row runs on the decode kernel, the one form that may split K across workgroups)
 size_t sbvr_hip_mm_T_workspace(int M, int N)
 {
-    return M > 0 && N > 0 ? static_cast<size_t>(M) * N * sizeof(unsigned long long) : 0;
+    return M == 1 && N > 0 ? static_cast<size_t>(N) * sizeof(unsigned long long) : 0;
 }
 
 int sbvr_hip_mm_T(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_bytes,
@@ -3918,6 +4016,77 @@ int sbvr_hip_mm_T_ws(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_b
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess)
         return fail(SBVR_HIP_ELAUNCH, "mm_T launch: %s", hipGetErrorString(e));
+    return SBVR_HIP_OK;
+}
+
+
+int sbvr_hip_read_floor(const void *buf, size_t buf_bytes, size_t bytes, int workgroups, int waves, int ahead, int pattern,
+                        int row_bytes, int win_bytes, void *sink, void *stream)
+{
+    if (!buf || !sink || reinterpret_cast<uintptr_t>(buf) % 16 != 0)
+        return fail(SBVR_HIP_EINVAL, "read floor: buffer and sink must be given, the buffer 16-byte aligned");
+    if (workgroups <= 0 || waves <= 0 || waves > 16 || ahead <= 0 || pattern < 0 || pattern > 2)
+        return fail(SBVR_HIP_EINVAL, "read floor: workgroups=%d waves=%d ahead=%d pattern=%d", workgroups, waves, ahead, pattern);
+    const size_t per_wave = bytes / 1024 / (static_cast<size_t>(workgroups) * waves);
+    if (per_wave == 0 || per_wave > 0x7ffffffeu || per_wave * workgroups * waves * 1024 != bytes || per_wave % ahead != 0)
+        return fail(SBVR_HIP_EINVAL, "read floor: %zu bytes are not a whole number of %d-KiB rounds for %d x %d waves",
+                    bytes, ahead, workgroups, waves);
+    if (pattern != 2) {
+        if (bytes > buf_bytes)
+            return fail(SBVR_HIP_EINVAL, "read floor: %zu bytes asked of a buffer of %zu", bytes, buf_bytes);
+    } else {
+        // rows of row_bytes, windows of win_bytes (whole 16 bytes), four rows per unit, the rows split over the waves
+        if (row_bytes <= 0 || row_bytes % 16 || win_bytes < 16 || win_bytes % 16 || static_cast<size_t>(workgroups) * win_bytes > static_cast<size_t>(row_bytes))
+            return fail(SBVR_HIP_EINVAL, "read floor: windows of %d bytes x %d workgroups do not fit rows of %d", win_bytes, workgroups, row_bytes);
+        const size_t tiles = (static_cast<size_t>(win_bytes) + 255) / 256;
+        if (per_wave % tiles)
+            return fail(SBVR_HIP_EINVAL, "read floor: %zu units per wave are not whole windows of %zu tiles", per_wave, tiles);
+        const size_t rows = per_wave / tiles * 4 * waves;
+        if (rows * static_cast<size_t>(row_bytes) > buf_bytes)
+            return fail(SBVR_HIP_EINVAL, "read floor: %zu rows of %d bytes reach beyond the buffer of %zu", rows, row_bytes, buf_bytes);
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid(static_cast<unsigned>(workgroups)), block(static_cast<unsigned>(64 * waves));
+    const v4u *b = static_cast<const v4u *>(buf);
+    uint32_t *sk = static_cast<uint32_t *>(sink);
+    const uint32_t u = static_cast<uint32_t>(per_wave);
+#define SBVR_RF(A) case A: hipLaunchKernelGGL(sbvr_read_floor_kernel<A>, grid, block, 0, st, b, u, pattern, \
+                                              static_cast<uint32_t>(row_bytes), static_cast<uint32_t>(win_bytes), sk); break
+    switch (ahead) {
+        SBVR_RF(1); SBVR_RF(2); SBVR_RF(3); SBVR_RF(4); SBVR_RF(7); SBVR_RF(8); SBVR_RF(14); SBVR_RF(16);
+    default: return fail(SBVR_HIP_EINVAL, "read floor: ahead must be one of 1, 2, 3, 4, 7, 8, 14, 16");
+    }
+#undef SBVR_RF
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return fail(SBVR_HIP_ELAUNCH, "read floor launch: %s", hipGetErrorString(e));
+    return SBVR_HIP_OK;
+}
+
+
+int sbvr_hip_decode_plan(int M, int N, int K, int S, int G, int cus, int *plan)
+{
+    if (!plan || cus <= 0)
+        return fail(SBVR_HIP_EINVAL, "decode plan: plan must be given and cus positive");
+    for (int i = 0; i < 8; ++i)
+        plan[i] = 0;
+    if (!mfma_path_ok(M, N, K, S, G))
+        return SBVR_HIP_OK;
+    if (batch_path_ok(M, N, K, S, G)) {
+        const BatchPlan p = plan_batch_uncached(M, N, K, S, cus);
+        if (p.CTW > 0) {
+            const int v[8] = {2, p.CTW, p.SP, p.MT, p.waves, p.n_wgs, p.ksplit, kMaxWaves};
+            for (int i = 0; i < 8; ++i)
+                plan[i] = v[i];
+            return SBVR_HIP_OK;
+        }
+    }
+    const GemvPlan p = plan_gemv_uncached(M, N, K, S, cus, 1);
+    if (p.CT > 0) {
+        const int v[8] = {1, p.CT, p.SP, p.MT, p.waves, p.n_wgs, p.ksplit, gemv_max_waves(p.MT, p.CT)};
+        for (int i = 0; i < 8; ++i)
+            plan[i] = v[i];
+    }
     return SBVR_HIP_OK;
 }
 

@@ -209,11 +209,13 @@ torch::Tensor sbvr_mm_T(torch::Tensor l_bvr, torch::Tensor l_coeff_idx, torch::T
     auto out = torch::empty({M, N}, torch::dtype(torch::kFloat16).device(l_bvr.device()));
     hipStream_t stream = current_stream();
     const size_t need = sbvr_hip_mm_T_workspace(static_cast<int>(M), static_cast<int>(N));
-    torch::Tensor ws = workspace(need, l_bvr, stream);
+    torch::Tensor ws;                    // (no split of K for this call: no workspace, nothing allocated)
+    if (need)
+        ws = workspace(need, l_bvr, stream);
     check(sbvr_hip_mm_T_ws(static_cast<const uint32_t *>(l_bvr.data_ptr()), l_coeff_idx.data_ptr(), lib,
                            l_coeff_cache.data_ptr(), static_cast<const uint32_t *>(r_bvr.data_ptr()), r_coeff_idx.data_ptr(),
                            rib, r_coeff_cache.data_ptr(), bias_ptr(bias, N, l_bvr), out.data_ptr(), M, N, K, Sl, Sr, G, Ll,
-                           Lr, ws.data_ptr(), need, stream));
+                           Lr, need ? ws.data_ptr() : nullptr, need, stream));
     return out;
 }
 
@@ -235,10 +237,12 @@ torch::Tensor sbvr_row_deq_mm_T(torch::Tensor l_w, torch::Tensor r_bvr, torch::T
     auto out = torch::empty({M, N}, torch::dtype(torch::kFloat16).device(l_w.device()));
     hipStream_t stream = current_stream();
     const size_t need = sbvr_hip_row_deq_mm_T_workspace(static_cast<int>(M), static_cast<int>(N));
-    torch::Tensor ws = workspace(need, l_w, stream);
+    torch::Tensor ws;                    // (no split of K for this call: no workspace, nothing allocated)
+    if (need)
+        ws = workspace(need, l_w, stream);
     check(sbvr_hip_row_deq_mm_T_ws(l_w.data_ptr(), static_cast<const uint32_t *>(r_bvr.data_ptr()), r_coeff_idx.data_ptr(), ib,
                                    r_coeff_cache.data_ptr(), bias_ptr(bias, N, l_w), out.data_ptr(), M, N, K, S, G, L,
-                                   ws.data_ptr(), need, stream));
+                                   need ? ws.data_ptr() : nullptr, need, stream));
     return out;
 }
 

@@ -117,6 +117,9 @@ class SbvrLlamaDecoder:
         self.head_ws = torch.zeros(2, dtype=torch.int64, device=dev)              # cross-workgroup argmax of the head kernel
         self.graph = None
         self.stream = torch.cuda.Stream(device=dev)
+        # probe(layer, residual): called by an eager fused step with the residual stream as it enters each layer
+        # (layer 0: the embedding row) and, as layer == layers, as it enters the final norm; for tests
+        self.probe = None
 
     # -- sizes ---------------------------------------------------------------
     def encoded_bytes(self):
@@ -162,13 +165,17 @@ class SbvrLlamaDecoder:
         a, b, ctx = self.x, self.x_alt, self.ctx
         torch.index_select(self.embed, 0, self.tok, out=a)            # (1, hidden)
         delta = self.zero
-        for layer in self.layers:
+        for number, layer in enumerate(self.layers):
             qkv = layer["qkv"].after_add_rmsnorm(a, delta, layer["norm1"], s.rms_eps, b)
+            if self.probe is not None:
+                self.probe(number, b)
             hip.dec_attention(qkv, self.cos, self.sin, self.pos, layer["k"], layer["v"], ctx,
                               s.heads, s.kv_heads, s.head_dim, self.rot_now)
             delta = layer["o"](ctx)
             gate_up = layer["gate_up"].after_add_rmsnorm(b, delta, layer["norm2"], s.rms_eps, a)
             delta = layer["down"].after_swiglu(gate_up)
+        if self.probe is not None:
+            self.probe(len(self.layers), (a.float() + delta.float()).to(torch.float16))
         if hip.dec_head_argmax_supported(s.hidden):
             # final norm, head, argmax and position advance in one launch
             hip.dec_head_argmax(a, delta, self.final_norm, s.rms_eps, self.lm_head, self.logits, self.tok,

@@ -44,6 +44,7 @@ def _load():
     lib.sbvr_hip_version.restype = i
     lib.sbvr_hip_last_error.restype = ctypes.c_char_p
     lib.sbvr_hip_last_kernel.restype = i
+    lib.sbvr_hip_last_rounding.restype = i
     lib.sbvr_hip_init.argtypes = [i]
     lib.sbvr_hip_linear_f16_workspace.restype = sz
     lib.sbvr_hip_linear_f16_workspace.argtypes = [i, i, i, i, i]
@@ -55,6 +56,7 @@ def _load():
     lib.sbvr_hip_linear_f16_stream_floor.argtypes = [vp, vp, i, vp, vp, i, i, i, i, i, vp, sz, vp]
     lib.sbvr_hip_row_deq_mm_T.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp]
     lib.sbvr_hip_row_deq_mm_T_ws.argtypes = [vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp, sz, vp]
+    lib.sbvr_hip_read_floor.argtypes = [vp, sz, sz, i, i, i, i, i, i, vp, vp]
     lib.sbvr_hip_row_deq_mm_T_workspace.restype = sz
     lib.sbvr_hip_row_deq_mm_T_workspace.argtypes = [i, i]
     lib.sbvr_hip_mm_T.argtypes = [vp, vp, i, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, i, i, vp]
@@ -85,6 +87,16 @@ KERNEL_PORTABLE, KERNEL_DECODE, KERNEL_ROWS32, KERNEL_PREFILL, KERNEL_PREFILL_SP
 def last_kernel():
     """Which kernel the last linear call of this thread launched (one of the KERNEL_* codes)."""
     return _load().sbvr_hip_last_kernel()
+
+
+ROUNDING_EXACT, ROUNDING_DECODE, ROUNDING_PLANEWISE = 1, 2, 3
+
+
+def last_rounding():
+    """How the last linear call of this thread treated the weights: ROUNDING_EXACT (no per-weight rounding),
+    ROUNDING_DECODE (each weight rounded to fp16 once, as the reference's decode() does) or ROUNDING_PLANEWISE
+    (an fp16 sum built plane by plane)."""
+    return _load().sbvr_hip_last_rounding()
 
 
 def _sbvr_hip_init(device=None):
@@ -249,6 +261,22 @@ def _sbvr_linear_f16_stream_floor(bvr, coeff_idx, coeff_cache, bvr_len=None, out
     return out
 
 
+_read_sinks = {}
+
+
+def read_floor(buf, nbytes, workgroups, waves, ahead, pattern=0, row_bytes=0, win_bytes=0):
+    """Measurement aid (``sbvr_hip_read_floor``): a launch of ``workgroups`` x ``waves`` waves that only reads
+    ``nbytes`` of the tensor ``buf``, 1 KiB per wave request, ``ahead`` requests of a wave in flight."""
+    lib = _load()
+    dev = buf.device
+    sink = _read_sinks.get(dev)
+    if sink is None:
+        sink = _read_sinks[dev] = torch.zeros(64, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _check(lib.sbvr_hip_read_floor(buf.data_ptr(), buf.numel() * buf.element_size(), nbytes, workgroups, waves,
+                                       ahead, pattern, row_bytes, win_bytes, sink.data_ptr(), _stream()))
+
+
 def _sbvr_row_deq_mm_T(l_w, r_bvr, r_coeff_idx, r_coeff_cache, bias, use_shfl=0, bvr_len=None):
     """fp16 ``l_w`` (M, K) against a ``trans=True`` weight: ``r_bvr`` (N/32, K, S),
     ``r_coeff_idx`` (N/G, K) (sbvr_ops.cpp:79-120).  ``use_shfl`` selected between
@@ -270,10 +298,10 @@ def _sbvr_row_deq_mm_T(l_w, r_bvr, r_coeff_idx, r_coeff_cache, bias, use_shfl=0,
     out = torch.empty((M, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         need = lib.sbvr_hip_row_deq_mm_T_workspace(M, N)
-        ws = _workspace(need, dev)
+        ws = _workspace(need, dev) if need else None          # (0: the call does not split K)
         _check(lib.sbvr_hip_row_deq_mm_T_ws(l_w.data_ptr(), r_bvr.data_ptr(), r_coeff_idx.data_ptr(), ib,
                                             r_coeff_cache.data_ptr(), _bias_ptr(bias, N, dev), out.data_ptr(),
-                                            M, N, K, S, G, L, ws.data_ptr(), need, _stream()))
+                                            M, N, K, S, G, L, ws.data_ptr() if need else None, need, _stream()))
     return out
 
 
@@ -300,12 +328,12 @@ def _sbvr_mm_T(l_bvr, l_coeff_idx, l_coeff_cache, r_bvr, r_coeff_idx, r_coeff_ca
     out = torch.empty((M, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         need = lib.sbvr_hip_mm_T_workspace(M, N)
-        ws = _workspace(need, dev)
+        ws = _workspace(need, dev) if need else None          # (0: the call does not split K)
         _check(lib.sbvr_hip_mm_T_ws(l_bvr.data_ptr(), l_coeff_idx.data_ptr(), _idx_bytes(l_coeff_idx, Ll, "l_coeff_idx"),
                                     l_coeff_cache.data_ptr(), r_bvr.data_ptr(), r_coeff_idx.data_ptr(),
                                     _idx_bytes(r_coeff_idx, Lr, "r_coeff_idx"), r_coeff_cache.data_ptr(),
                                     _bias_ptr(bias, N, dev), out.data_ptr(), M, N, K, Sl, Sr, G, Ll, Lr,
-                                    ws.data_ptr(), need, _stream()))
+                                    ws.data_ptr() if need else None, need, _stream()))
     return out
 
 

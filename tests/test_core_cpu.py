@@ -166,10 +166,45 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in sbvr_hip.h but not exported"
     lib.sbvr_hip_version.restype = ctypes.c_int
-    assert lib.sbvr_hip_version() == 102
+    assert lib.sbvr_hip_version() == 103
     lib.sbvr_hip_linear_f16_workspace.restype = ctypes.c_size_t
     assert lib.sbvr_hip_linear_f16_workspace(1, 14336, 4096, 4, 128) == 14336 * 8
     assert lib.sbvr_hip_linear_f16_workspace(1, 64, 96, 4, 32) == 0        # portable kernel: no workspace
+
+
+def test_workspace_sizes_follow_the_split_predicates():
+    """The alternates' workspace queries ask for accumulators only where their launch may split K."""
+    import ctypes
+    from sbvr import hip
+    lib = hip._load()
+    assert lib.sbvr_hip_mm_T_workspace(1, 4096) == 4096 * 8           # one left row: the decode kernel, may split
+    assert lib.sbvr_hip_mm_T_workspace(2048, 14336) == 0              # more left rows never split
+    assert lib.sbvr_hip_row_deq_mm_T_workspace(1, 4096) == 4096 * 8   # 64 column workgroups on 256 CUs: split
+    assert lib.sbvr_hip_row_deq_mm_T_workspace(2048, 14336) == 0      # prefill-sized: the columns fill the device
+
+
+def test_decode_plans_respect_the_launch_bounds():
+    """Every launch shape the planners pick for up to 16 rows stays within the waves its kernel
+    instance is compiled for (a launch beyond them fails), over a grid of shapes and device sizes."""
+    import ctypes
+    from sbvr import hip
+    lib = hip._load()
+    plan = (ctypes.c_int * 8)()
+    seen = 0
+    for cus in (64, 228, 256, 304):
+        for M in (1, 2, 4, 5, 8, 9, 12, 16):
+            for N in (16, 48, 512, 1024, 4096, 6144, 14336, 28672, 128256):
+                for K in (128, 512, 2048, 4096, 8192, 14336):
+                    for S in (2, 3, 4, 6, 8):
+                        assert lib.sbvr_hip_decode_plan(M, N, K, S, 128, cus, plan) == 0
+                        kind, ct, sp, mt, waves, wgs, ksplit, bound = list(plan)
+                        if kind == 0:
+                            continue
+                        seen += 1
+                        assert 1 <= waves <= bound, (cus, M, N, K, S, list(plan))
+                        assert mt == (1 if M <= 4 else 2 if M <= 8 else 4), (M, list(plan))
+                        assert wgs >= 1 and 1 <= ksplit <= 255 and ct >= 1 and sp >= 1
+    assert seen > 4000
 
 
 def test_argument_validation_without_gpu():

@@ -14,6 +14,8 @@ import numpy as np
 import pytest
 import torch
 
+import parity
+
 pytestmark = pytest.mark.gpu
 
 
@@ -33,14 +35,12 @@ def check(y_gpu, yd, what=""):
     return rel.max(), ulp.max()
 
 
-def check_rounded(y_gpu, yd, what=""):
-    """The 32-row kernel (9..32 rows by default) rounds each decoded weight to fp16, as the reference's decode()
-    does: at most 3e-3 of the RMS output off, 1e-2 relative for outputs above 0.3 RMS."""
-    y = y_gpu.float().cpu().numpy().astype(np.float64)
-    rms = float(np.sqrt(np.mean(yd ** 2))) + 1e-30
-    err = np.abs(y - yd)
-    assert err.max() <= 3e-3 * rms + 2.0 ** -11 * np.abs(yd).max(), f"{what}: error {err.max() / rms:.3e} of the RMS output"
-    assert (err / np.maximum(np.abs(yd), 0.3 * rms)).max() <= 1e-2, what
+def check_rounded(oracle, y_gpu, yd, operands, rounding, what=""):
+    """The 32-row kernel (9..32 rows by default) rounds each decoded weight to fp16: in its table look-up form
+    exactly as the reference's decode() does, which the oracle's mode 1 restates (tests/parity.py)."""
+    x, bn, inn, cache, G = operands
+    _, yd1 = oracle.C.linear_f16(x, bn, inn, cache, G, mode=1)
+    return parity.judge(y_gpu.float().cpu().numpy(), yd, yd1, rounding, what)
 
 
 DECODE, ROWS32 = 2, 3
@@ -59,7 +59,7 @@ def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False, flags=0, sigma=0.02, 
     y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev),
                               None if b is None else b.to(dev), bvr_len=G, flags=flags)
     torch.cuda.synchronize()
-    ran = hip.last_kernel()
+    ran, rounding = hip.last_kernel(), hip.last_rounding()
     if flags == 2 and M <= 16:
         assert ran != ROWS32 or G % 128 != 0 or N < 16, f"flags=2 ran kernel {ran}"
     bn, inn, bb = bvr.numpy(), idx.numpy(), None if b is None else b.numpy()
@@ -82,7 +82,8 @@ def run_case(oracle, N, K, S, G, M, L, seed=0, bias=False, flags=0, sigma=0.02, 
         assert diff.max() <= 2.0 ** -9 * max(np.abs(yd).max(), rms), f"bias case off by {diff.max()}"
         return
     if ran == ROWS32:
-        return check_rounded(y, yd, f"N={N} K={K} S={S} G={G} M={M} L={L} flags={flags} (32-row kernel)")
+        return check_rounded(oracle, y, yd, (x.numpy(), bn, inn, cache.numpy(), G), rounding,
+                             f"N={N} K={K} S={S} G={G} M={M} L={L} flags={flags} (32-row kernel)")
     return check(y, yd, f"N={N} K={K} S={S} G={G} M={M} L={L} flags={flags}")
 
 
@@ -202,15 +203,20 @@ def test_batch_rows_of_different_magnitude(oracle):
     x[5] = 0.0
     x[9] *= 1e-3
     x = x.to(torch.float16)
+    from sbvr import hip
     _, yd = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), G)
-    # flags = 2: the decode kernel of 5..16 rows (exact); default: the 32-row kernel (weights rounded to fp16)
-    for flags, judge in ((2, check), (0, check_rounded)):
+    _, yd1 = oracle.C.linear_f16(x.numpy(), bvr.numpy(), idx.numpy(), cache.numpy(), G, mode=1)
+    # flags = 2: the decode kernel of 5..16 rows (exact); default: the 32-row kernel (weights rounded to fp16 as
+    # decode() rounds them)
+    for flags, rounding in ((2, parity.ROUNDING_EXACT), (0, parity.ROUNDING_DECODE)):
         y = sbvr._sbvr_linear_f16(x.to(dev), bvr.to(dev), idx.to(dev), cache.to(dev), None, bvr_len=G, flags=flags)
+        assert hip.last_rounding() == rounding
+        got = y.float().cpu().numpy()
         for m in range(M):           # row by row: each against its own RMS
             if m == 5:
                 assert float(y[m].float().abs().max()) == 0.0
             else:
-                judge(y[m:m + 1], yd[m:m + 1], f"row {m}, flags {flags}")
+                parity.judge(got[m:m + 1], yd[m:m + 1], yd1[m:m + 1], rounding, f"row {m}, flags {flags}")
 
 
 def test_batch_rows_repeatable(oracle):

@@ -69,9 +69,40 @@ def test_noalloc_equals_workspace_entry_point(oracle):
     big = case(256, 1024, 4, 48, 256, 33, False)
     assert torch.equal(_call(lib, "noalloc", *big, 128), _call(lib, "workspace", *big, 128, ws=ws))
 
-    # beyond the array: refused with a clear error, nothing launched
-    x, bvr, idx, cache, _ = case(64, 128, 2, 1, 16, 34, False)
+    # Beyond the array (M * N > 524288).  Every buffer below has its real size: whichever way the call goes, no
+    # kernel reads or writes out of bounds.
+    def device_case(N, K, S, M, seed):
+        gen = torch.Generator(device=dev).manual_seed(seed)
+        bvr = torch.randint(-2 ** 31, 2 ** 31, (K // 32, N, S), dtype=torch.int32, generator=gen, device=dev).view(torch.uint32)
+        idx = torch.randint(0, 16, (K // 128, N), dtype=torch.int32, generator=gen, device=dev).to(torch.uint8)
+        cache = synth.make_lines(16, S, 0.02, seed).to(dev)
+        x = torch.randn((M, K), generator=gen, device=dev).to(torch.float16)
+        return x, bvr, idx, cache
+
+    plan = (ctypes.c_int * 8)()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # (a) a decode launch that cannot do without the split of K (8 rows, K = 14336: a workgroup covers at most
+    #     a seventh of K): refused with a clear error, nothing launched
+    M, N, K, S = 8, 70016, 14336, 2
+    assert lib.sbvr_hip_decode_plan(M, N, K, S, 128, cus, plan) == 0
+    assert plan[0] != 0 and plan[6] > 1, f"this shape is expected to split K across workgroups: {list(plan)}"
+    x, bvr, idx, cache = device_case(N, K, S, M, 34)
+    out = torch.full((M, N), float("nan"), dtype=torch.float16, device=dev)
     rc = lib.sbvr_hip_linear_f16_noalloc(x.data_ptr(), bvr.data_ptr(), idx.data_ptr(), 1, cache.data_ptr(), None,
-                                         x.data_ptr(), 16, 40000, 128, 2, 128, 16, 0, stream)
-    assert rc == -4 and b"noalloc" in lib.sbvr_hip_last_error()
+                                         out.data_ptr(), M, N, K, S, 128, 16, 0, stream)
+    assert rc == -4 and b"noalloc" in lib.sbvr_hip_last_error(), (rc, lib.sbvr_hip_last_error())
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(out.float()).all()), "a refused call wrote to its output"
+    del x, bvr, idx, cache, out
+    # (b) 16 rows of 40000 columns: the table look-up kernel, which runs unsplit without accumulators: not refused,
+    #     and equal to the workspace entry point up to the order of the fp32 additions (that one may split K)
+    M, N, K, S = 16, 40000, 1024, 2
+    x, bvr, idx, cache = device_case(N, K, S, M, 35)
+    big_ws = torch.zeros(M * N * 8, dtype=torch.uint8, device=dev)
+    got = _call(lib, "noalloc", x, bvr, idx, cache, None, 128)
+    want = _call(lib, "workspace", x, bvr, idx, cache, None, 128, ws=big_ws)
+    assert not torch.isnan(got.float()).any()
+    rms = float(want.float().pow(2).mean().sqrt())
+    assert float((got.float() - want.float()).abs().max()) <= 2.0 ** -9 * max(rms, float(want.float().abs().max()))
+    assert int(big_ws.max()) == 0
