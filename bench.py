@@ -316,15 +316,16 @@ def sweep_leg():
     dev = torch.device("cuda:0")
     rows = []
 
-    def one(n, k, s, m, tag):
+    def one(n, k, s, m, tag, g=GROUP, lines=LINES):
         per = n * k * s // 8
         copies = max(2, min(16, int(600e6 // per)))
-        ws = [tuple(t.to(dev) for t in synth.random_encoding(n, k, s, GROUP, LINES, seed=c)) for c in range(copies)]
+        ws = [tuple(t.to(dev) for t in synth.random_encoding(n, k, s, g, lines, seed=c)) for c in range(copies)]
         x = torch.randn((m, k), generator=torch.Generator().manual_seed(5)).to(torch.float16).to(dev)
         out = torch.empty((m, n), dtype=torch.float16, device=dev)
-        t = _graph_time(lambda i: hip._sbvr_linear_f16(x, *ws[i % copies], None, GROUP, out=out), 100)
-        nbytes = algorithmic_bytes(n, k, s, GROUP, LINES, m)
-        rows.append({"linear": tag, "N": n, "K": k, "S": s, "M": m, "us": round(t * 1e6, 2),
+        t = _graph_time(lambda i: hip._sbvr_linear_f16(x, *ws[i % copies], None, g, out=out), 100)
+        nbytes = algorithmic_bytes(n, k, s, g, lines, m)
+        rows.append({"linear": tag, "N": n, "K": k, "S": s, "M": m, "G": g, "lines": lines,
+                     "idx": "uint8" if lines <= 256 else "uint16", "us": round(t * 1e6, 2),
                      "GBps": round(nbytes / t / 1e9, 1), "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4)})
         del ws
         torch.cuda.empty_cache()
@@ -332,6 +333,15 @@ def sweep_leg():
     for tag, n, k in (("q/o", 4096, 4096), ("k/v", 1024, 4096), ("q|k|v", 6144, 4096), ("gate/up", 14336, 4096),
                       ("gate|up", 28672, 4096), ("down", 4096, 14336)):
         one(n, k, 4, 1, tag)
+    # tables of more than 256 lines, hence uint16 line indices (the reference switches the index width at
+    # L = 256, sbvr_kernel.cu:931-932): config 1 and the gate shape with 300 lines, and the fused matrices of the
+    # decoder with the tables they really carry (three and two tables of 256 lines one behind the other)
+    for tag, n, k, lines in (("q/o", 4096, 4096, 300), ("gate/up", 14336, 4096, 300), ("q|k|v", 6144, 4096, 768),
+                             ("gate|up", 28672, 4096, 512)):
+        one(n, k, 4, 1, tag, lines=lines)
+    # the reference's own group length of 256 elements (sbvr/core.py:222) at the four layer shapes
+    for tag, n, k in (("q/o", 4096, 4096), ("k/v", 1024, 4096), ("gate/up", 14336, 4096), ("down", 4096, 14336)):
+        one(n, k, 4, 1, tag, g=256)
     for tag, n, k in (("gate", 14336, 4096), ("down", 4096, 14336)):
         for s in (2, 3, 4):
             for m in (1, 2, 4, 8, 16):
@@ -556,6 +566,12 @@ def main():
         "frac_of_hbm_peak": round(nbytes / (floor_t["median_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
     }
     wall_ms, timing, launcher, device = gpu_leg(a.steps, a.warmup)
+    global _WEIGHTS
+    _WEIGHTS = None                      # (the legs below want the memory)
+    reads = read_floor_leg(quick=True)
+    read_floor = dict(reads["best"], what="the fastest of a few launches that only read the gate shape's 28 MiB of plane words "
+                                          "(sbvr_hip_read_floor; python bench.py --read-floor runs the whole grid of shapes)")
+    read_floor["us_for_the_workload_bytes"] = round(nbytes / (read_floor["GBps"] * 1e9) * 1e6, 3)
     if a.stream_floor:
         print(json.dumps({"metric": "SBVR gate GEMV 4096->14336: kernel and its memory-request floor, us per launch",
                           "kernel_us": round(timing["median_ms"] * 1e3, 3), "kernel_us_min": round(timing["min_ms"] * 1e3, 3),
@@ -604,10 +620,10 @@ def main():
             "traffic_source": TRAFFIC_PROFILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this "
                               "command, scaled by a 256 MiB copy; not measured in this run)",
             "stream_floor": floor,
+            "read_floor": read_floor,
+            "kernel_over_read_floor": round(timing["median_ms"] * 1e3 / read_floor["us_for_the_workload_bytes"], 3),
         },
     }
-    global _WEIGHTS
-    _WEIGHTS = None                      # (the decode leg wants the memory)
     if not a.no_decode:
         line["decode"] = decode_leg()
     if not a.no_cpu:

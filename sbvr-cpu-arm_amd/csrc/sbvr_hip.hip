@@ -154,6 +154,7 @@ constexpr int kSub = 128;        // K elements per MFMA (one sub-group)
 constexpr int kMaxWaves = 16;    // waves of a workgroup; they split K among themselves
 constexpr int kMaxM = 16;        // batch rows of the decode kernel (row tiles of 4)
 constexpr int kUnitsAhead = 3;   // units of plane words a wave of the decode kernel keeps in flight
+constexpr int kUnitsFirst = 2;   // of those, requested before the wave makes its A operands (the rest right behind them)
 constexpr float kLastTermScale = 256.f;  // third fp8 term of an activation holds residual * 256
 
 // Split-K accumulator: one 64-bit word per output, [count:8 | sum:56].  Every
@@ -566,7 +567,12 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
     // (workgroups of at most 8 waves keep twice as many, for the same number of requests per CU)
     constexpr int kAhead = gemv_max_waves(MT, CT) == 8 ? 2 * kUnitsAhead : kUnitsAhead;
     constexpr int kPre = U < kAhead ? U : kAhead;
-    request_units(0, kPre);
+    // Only kUnitsFirst of them before the operands are made, the rest right behind them: with every wave's full
+    // share asked for at once the CU's queue is full when its youngest waves come to ask for their activations,
+    // and those waves then start their units a microsecond and more behind the oldest (4096 -> 14336: 7.8 -> 7.5 us;
+    // one unit first was slower again).
+    constexpr int kPre0 = kUnitsFirst * (kAhead / kUnitsAhead) < kPre ? kUnitsFirst * (kAhead / kUnitsAhead) : kPre;
+    request_units(0, kPre0);
     __builtin_amdgcn_sched_barrier(0);       // these requests are out before anything waits
     SBVR_STAMP(1);
 
@@ -683,7 +689,8 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
         }
     };
     make_operands(0, SP);
-    __builtin_amdgcn_s_setprio(0);
+    request_units(kPre0, kPre);
+    __builtin_amdgcn_sched_barrier(0);
     SBVR_STAMP(2);
 
     // -- 3. coefficient lines (S fp16 each): lane l gathers the line of column n_base + l for each
@@ -737,6 +744,17 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int sgi = u / CT;
+        // A wave's priority falls as it gets through its units (3 for the first quarter down to 0 for the last): the
+        // CU gives its instruction slots and the free places of its memory queue to the oldest wave among equals,
+        // so with one priority for all the youngest waves of a workgroup finished their units 2 us after the oldest,
+        // which then sat at the barrier below (median wait 1.2 us, 0.6 us with this; 7.5 -> 7.4 us at 4096 -> 14336).
+        if (u == 0 || (u * 4) / U != ((u - 1) * 4) / U)
+            switch (3 - (u * 4) / U) {               // (u is a constant once the loop is unrolled)
+            case 3: __builtin_amdgcn_s_setprio(3); break;
+            case 2: __builtin_amdgcn_s_setprio(2); break;
+            case 1: __builtin_amdgcn_s_setprio(1); break;
+            default: __builtin_amdgcn_s_setprio(0); break;
+            }
         request_units(u + kPre, u + kPre + 1);      // keeps kPre units of this wave in flight
         if (u > 0)
             fetch_coefficients(u - 1);              // (on its way while this unit's operands are made)
@@ -769,6 +787,7 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
             }
         __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_s_setprio(0);
     fetch_coefficients(U - 1);
     apply_coefficients(U - 1);
     SBVR_STAMP(4);
