@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the gate GEMV as the hardware counters saw them: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy.  A profiler run's figure,
 # not measured by this script: the line names the file it comes from.
-TRAFFIC_FROM_PROFILE_BYTES = 30.09e6
+TRAFFIC_FROM_PROFILE_BYTES = 30.07e6
 TRAFFIC_PROFILE = "profiles/sbvr_gemv_mfma_gate_4096x14336.txt"
 MIN_TIMED_LAUNCHES = 200
 _WEIGHTS = None        # the rotating weight copies on the device (built once per process)
@@ -307,10 +307,11 @@ def read_floor_leg(quick=False):
     return out
 
 
-def sweep_leg():
+def sweep_leg(only=None):
     """The other decode configurations of the reference's benchmark plan: every linear of a
     Llama-3-8B layer at batch 1, and gate / down at batch 1..16 with 2, 3 and 4 planes.
-    Weights rotate through enough copies to exceed the 256 MB Infinity Cache."""
+    Weights rotate through enough copies to exceed the 256 MB Infinity Cache.
+    only = (N, K, M): that one linear alone (4 planes, groups of 128, 256 lines), e.g. under a profiler."""
     import torch
     from sbvr import synth, hip
     dev = torch.device("cuda:0")
@@ -330,6 +331,9 @@ def sweep_leg():
         del ws
         torch.cuda.empty_cache()
 
+    if only is not None:
+        one(only[0], only[1], 4, only[2], "%dx%d" % (only[0], only[1]))
+        return rows
     for tag, n, k in (("q/o", 4096, 4096), ("k/v", 1024, 4096), ("q|k|v", 6144, 4096), ("gate/up", 14336, 4096),
                       ("gate|up", 28672, 4096), ("down", 4096, 14336)):
         one(n, k, 4, 1, tag)
@@ -519,6 +523,8 @@ def main():
     ap.add_argument("--decode-only", action="store_true", help="run only the 8B decode leg and print its figures")
     ap.add_argument("--sweep", action="store_true",
                     help="run only the layer-shape / batch / plane-count sweep of the decode kernel and print it")
+    ap.add_argument("--shape", default=None, metavar="NxK[xM]",
+                    help="run only the linear of this shape (4 planes, groups of 128, batch M, default 1) and print it")
     ap.add_argument("--prefill", action="store_true", help="run only the prefill GEMM sizes and print them")
     ap.add_argument("--other-ops", action="store_true",
                     help="run only _sbvr_mm_T and _sbvr_row_deq_mm_T at the layer shapes and print them")
@@ -537,6 +543,11 @@ def main():
 
     if a.decode_only:
         print(json.dumps({"metric": "8B decode tokens/s", "decode": decode_leg()}))
+        return
+    if a.shape:
+        dims = [int(v) for v in a.shape.lower().split("x")]
+        only = (dims[0], dims[1], dims[2] if len(dims) > 2 else 1)
+        print(json.dumps({"metric": "SBVR decode linear, us and GB/s of algorithmic bytes", "sweep": sweep_leg(only)}))
         return
     if a.sweep:
         print(json.dumps({"metric": "SBVR decode linears, us and GB/s of algorithmic bytes", "sweep": sweep_leg()}))
