@@ -113,10 +113,15 @@ size_t sbvr_hip_linear_f16_workspace(int M, int N, int K, int S, int G);
  *                   otherwise the one that decodes weight tiles into LDS; same
  *                   results up to the order of the fp32 additions;
  *   portable kernel everything else (one thread per output), and with flags bit 0.
- * The 32-row and prefill kernels decode the weights to fp16 first (each decoded
- * weight an fp16 sum of its coefficients, as decode() of sbvr/core.py:927-949
- * rounds weights to fp16): their error is a few 1e-3 of the RMS output, within
- * the 1e-2 relative bound for outputs that are not small against it.
+ * The 32-row and prefill kernels decode the weights to fp16 first.  Their table
+ * look-up forms (2..4 planes) round the sum of a weight's coefficients once,
+ * which is how decode() of sbvr/core.py:927-949 produces a weight (bin_combs @
+ * coeff, :345-366): against x @ decode(W)^T they are as close as the decode
+ * kernel is to the unrounded weights (2 fp16 ulps).  Their arithmetic forms (6
+ * and 8 planes, groups of 32 or 64) add the coefficients up in fp16 plane by
+ * plane.  Either way the error against unrounded weights is a few 1e-3 of the
+ * RMS output, within the 1e-2 relative bound for outputs that are not small
+ * against it.  sbvr_hip_last_rounding() tells which of the three a call took.
  * The reference has no kernel of exactly this form (its fp16-activation
  * kernels, sbvr_kernel.cu:121-359 behind sbvr_ops.cpp:79-120, want the
  * trans=True layout); this is the operator its models/sbvr_llama.py:86-87

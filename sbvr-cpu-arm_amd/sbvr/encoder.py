@@ -9,7 +9,11 @@ same lines and selectors.  On a GPU two things differ from the reference's loop
 (core.py:711-722, one group at a time):
   * the error of a (group, line) pair comes from a HIP kernel that keeps the
     (lines, G, 2^S) tensor of squared differences in registers (hip.encoder_group_mse;
-    fp16 compute type and S <= 6, otherwise the torch expression);
+    fp16 compute type and up to 8 planes, otherwise the torch expression).  The kernel
+    sums a group's minima in fp32 in element order where torch's .mean() reduces in
+    another order, so on near-ties a GPU run can pick another line than a CPU run
+    (parity of GPU encodings with the reference's own GPU runs is unpinned; they are
+    compared by their error);
   * table look-ups run for a block of groups at once (``encode_all``): the
     groups of a block are looked up against the table as it stands, the leading
     hits are taken, the first miss goes through the one-group path (which may add
