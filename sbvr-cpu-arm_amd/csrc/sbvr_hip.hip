@@ -744,12 +744,13 @@ sbvr_gemv_mfma_kernel(const GemvArgs a)
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const int sgi = u / CT;
-        // A wave's priority falls as it gets through its units (3 for the first quarter down to 0 for the last): the
-        // CU gives its instruction slots and the free places of its memory queue to the oldest wave among equals,
-        // so with one priority for all the youngest waves of a workgroup finished their units 2 us after the oldest,
-        // which then sat at the barrier below (median wait 1.2 us, 0.6 us with this; 7.5 -> 7.4 us at 4096 -> 14336).
+        // A wave's priority falls as it gets through its units (2, 2, 1, 0 over their quarters, below the 3 of a
+        // wave that is making its operands): the CU gives its instruction slots and the free places of its memory
+        // queue to the oldest wave among equals, so with one priority for all the youngest waves of a workgroup
+        // finished their units 2 us after the oldest, which then sat at the barrier below (median wait 1.2 us, 0.6 us
+        // with this; 7.5 -> 7.4 us at 4096 -> 14336).
         if (u == 0 || (u * 4) / U != ((u - 1) * 4) / U)
-            switch (3 - (u * 4) / U) {               // (u is a constant once the loop is unrolled)
+            switch ((0x2210 >> (4 * (3 - (u * 4) / U))) & 0xf) {               // (u is a constant once the loop is unrolled)
             case 3: __builtin_amdgcn_s_setprio(3); break;
             case 2: __builtin_amdgcn_s_setprio(2); break;
             case 1: __builtin_amdgcn_s_setprio(1); break;
@@ -930,7 +931,10 @@ sbvr_gemv_batch_kernel(const GemvArgs a)
             }
     };
     constexpr int kPre = U < kUnitsAhead ? U : kUnitsAhead;
-    request_units(0, kPre);
+    // (one unit before the operands are made, the others right behind them, and the priority ladder of the kernel
+    // above over the units: 12.0 -> 11.4 us at 8 rows of 4096 -> 14336, 12.1 -> 11.4 at 14336 -> 4096)
+    constexpr int kPre0 = 1;
+    request_units(0, kPre0);
     __builtin_amdgcn_sched_barrier(0);
     SBVR_STAMP(1);
 
@@ -973,7 +977,8 @@ sbvr_gemv_batch_kernel(const GemvArgs a)
                 scl[slot * 4 + r] = row_scale;
         }
     }
-    __builtin_amdgcn_s_setprio(0);
+    request_units(kPre0, kPre);
+    __builtin_amdgcn_sched_barrier(0);
     SBVR_STAMP(7);
     __syncthreads();
     SBVR_STAMP(2);
@@ -1010,6 +1015,12 @@ sbvr_gemv_batch_kernel(const GemvArgs a)
 #pragma unroll
         for (int t = 0; t < CTW; ++t) {
             const int u = sgi * CTW + t;
+            if (u == 0 || (u * 4) / U != ((u - 1) * 4) / U)
+                switch ((0x2210 >> (4 * (3 - (u * 4) / U))) & 0xf) {
+                case 2: __builtin_amdgcn_s_setprio(2); break;
+                case 1: __builtin_amdgcn_s_setprio(1); break;
+                default: __builtin_amdgcn_s_setprio(0); break;
+                }
             request_units(u + kPre, u + kPre + 1);
             float c[S];
             {
@@ -1056,6 +1067,7 @@ sbvr_gemv_batch_kernel(const GemvArgs a)
         }
     }
 
+    __builtin_amdgcn_s_setprio(0);
     SBVR_STAMP(4);
     // -- 5. partial results meet in LDS; summed over the groups in a fixed order
     constexpr int kBlocks = CTW * MT;                 // (tile, row tile) blocks of a wave
@@ -1178,23 +1190,20 @@ GemvPlan plan_gemv_uncached(int M, int N, int K, int S, int cus, int min_waves)
     const EnvSwitches &env = env_switches();
     const int eCT = env.ct, eSP = env.sp, eW = env.waves;
     GemvPlan best{};
-    // (with the add + norm prologue the waves of a workgroup meet at a barrier before their operands: 8-wave
-    // workgroups with four sub-groups a wave measured 14.1-14.7 us against 16.0 for 16 waves with two at
-    // 4096 -> 28672, and only that large a matrix gains from taking all of K into the workgroup)
-    const bool norm = min_waves > 1;
-    const int wg_waves = norm ? 8 : std::min(kMaxWaves, gemv_max_waves(MT, 0));      // (never above the kernel's launch bound)
-    if (best.CT == 0 && eCT <= 0 && nsub % wg_waves == 0 && wg_waves >= min_waves && N >= (norm ? 64 : 16) * cus) {
+    // (the add + norm prologue, min_waves > 1, takes the same shapes: its barrier falls while the first units are in
+    // flight; 4096 -> 28672 with it 12.4 us as 256 x 16 waves against 14.9 us as 512 x 8 waves of four sub-groups)
+    const int wg_waves = std::min(kMaxWaves, gemv_max_waves(MT, 0));      // (never above the kernel's launch bound)
+    if (best.CT == 0 && eCT <= 0 && nsub % wg_waves == 0 && wg_waves >= min_waves && N >= 16 * cus) {
         const int SP = nsub / wg_waves;
-        // windows of wstride columns, r workgroups per CU; without the prologue one workgroup per CU takes up
-        // to 7 tiles (4096 -> 28672: 256 windows of 112 columns 11.8 us, 512 of 56 columns 13.1-13.5 us; with
-        // the prologue, whose barrier 16 waves feel more than 8, the two measured the same)
-        const int widest = norm ? 64 : 112;
+        // windows of wstride columns, r workgroups per CU; one workgroup per CU takes up to 7 tiles (4096 -> 28672:
+        // 256 windows of 112 columns 11.8 us, 512 of 56 columns 13.1-13.5 us)
+        const int widest = 112;
         for (int r = (N + widest * cus - 1) / (widest * cus); r <= 4; ++r) {
             const int wstride = ((N + cus * r - 1) / (cus * r) + 7) / 8 * 8;
             const int CT = (wstride + 15) / 16;
             if (wstride < 16)
                 break;
-            if (!has_instance(CT, SP) || !shape_ok_for(MT, CT, SP) || SP > (norm ? 4 : 2 * CT) || CT * 16 > N)
+            if (!has_instance(CT, SP) || !shape_ok_for(MT, CT, SP) || SP > 2 * CT || CT * 16 > N)
                 continue;
             best = GemvPlan{CT, SP, MT, wg_waves, (N + wstride - 1) / wstride, 1, 0, wstride};
             break;
@@ -2318,7 +2327,15 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
     line = load_line(p_begin + (kShare ? 2 : 1));
     // (the fences keep the loads of the next step in front of this step's arithmetic: left alone, the scheduler
     // moves them down to their first use, to save registers, and every step waits for loads it has just issued)
+    // (a wave's priority falls with its progress, as in the decode kernels: the CU serves the oldest wave among
+    // equals, and the youngest waves of a workgroup would finish last; 2-3 % at the 4096 <-> 14336 shapes)
+    const int l_quarter = ((p_end - p_begin) / 4 + 1) / 2 * 2;
+    __builtin_amdgcn_s_setprio(2);
     for (int ip = p_begin; ip < p_end; ip += 2) {
+        if (ip == p_begin + 2 * l_quarter)
+            __builtin_amdgcn_s_setprio(1);
+        if (ip == p_begin + 3 * l_quarter)
+            __builtin_amdgcn_s_setprio(0);
         load_step(ip + 1, s1, line, !kShare);
         if constexpr (!kShare)
             line = load_line(ip + 2);
@@ -2337,6 +2354,7 @@ sbvr_gemm_rows32_lut_kernel(const RowsArgs a)
         __builtin_amdgcn_sched_barrier(0);
     }
 
+    __builtin_amdgcn_s_setprio(0);
     // ---- partial results meet in LDS; D[i][jj] sits in lane jj + 32*((i/4)%2), register (i%4) + 4*(i/8)
 #pragma unroll
     for (int r = 0; r < 16; ++r)
