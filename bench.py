@@ -192,20 +192,31 @@ def decode_breakdown(dec):
         a, b, ctx, delta = dec.x, dec.x_alt, dec.ctx, dec.zero
         for layer in dec.layers:
             layer["qkv"].after_add_rmsnorm(a, delta, layer["norm1"], s.rms_eps, b)
-            delta = layer["o"](ctx)
+            if not dec.attention_o:
+                delta = layer["o"](ctx)
             gate_up = layer["gate_up"].after_add_rmsnorm(b, delta, layer["norm2"], s.rms_eps, a)
             delta = layer["down"].after_swiglu(gate_up)
 
     def attention():
         for layer in dec.layers:
-            hip.dec_attention(layer["qkv"].out, dec.cos, dec.sin, dec.pos, layer["k"], layer["v"], dec.ctx,
-                              s.heads, s.kv_heads, s.head_dim, dec.rot_now)
+            if dec.attention_o:
+                o = layer["o"]
+                hip.dec_attention_o(layer["qkv"].out, dec.cos, dec.sin, dec.pos, layer["k"], layer["v"], s.heads,
+                                    s.kv_heads, s.head_dim, o.bvr, o.idx, o.cache, None, o.bvr_len, out=o.out,
+                                    rot_now=dec.rot_now)
+            else:
+                hip.dec_attention(layer["qkv"].out, dec.cos, dec.sin, dec.pos, layer["k"], layer["v"], dec.ctx,
+                                  s.heads, s.kv_heads, s.head_dim, dec.rot_now)
 
     def head():
         hip.dec_head_argmax(dec.x, dec.zero, dec.final_norm, s.rms_eps, dec.lm_head, dec.logits, dec.tok,
                             dec.generated, dec.pos, dec.head_ws, dec.cos, dec.sin, dec.rot_now)
 
-    parts = {"linears (4 per layer, prologues folded in)": linears, "attention (1 per layer)": attention}
+    if dec.attention_o:
+        parts = {"linears (3 per layer, prologues folded in)": linears,
+                 "attention + o projection (1 launch per layer)": attention}
+    else:
+        parts = {"linears (4 per layer, prologues folded in)": linears, "attention (1 per layer)": attention}
     if hip.dec_head_argmax_supported(s.hidden):
         parts["final norm + fp16 head + argmax"] = head
     out = {}

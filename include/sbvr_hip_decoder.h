@@ -4,10 +4,14 @@
  *
  * All tensors are device pointers, fp16 unless stated (n even, head_dim 64 or 128), and the
  * launches go to `stream` (a hipStream_t, NULL = default stream).  Return
- * values: 0 ok, -1 invalid argument, -2 unsupported shape, -3 launch error.
+ * values: 0 ok, -1 invalid argument, -2 unsupported shape, -3 launch error,
+ * -4 workspace missing or too small.
  */
 #ifndef SBVR_HIP_DECODER_H
 #define SBVR_HIP_DECODER_H
+
+#include <stddef.h>
+#include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -37,6 +41,42 @@ int sbvr_hip_dec_add_rmsnorm_f16(void *x, const void *delta, const void *weight,
 int sbvr_hip_dec_attention_f16(const void *qkv, const float *cos_table, const float *sin_table, const float *rot_now,
                                const long long *pos, void *kcache, void *vcache, void *ctx, int heads, int kv_heads,
                                int head_dim, int max_seq, void *stream);
+
+/* sbvr_hip_dec_attention_f16 followed by the SBVR-encoded output projection
+ * (sbvr_hip_linear_f16 of the context row, sbvr_hip.h) in one launch:
+ * out[N] <- o_proj(attention(qkv)), i.e. `attn_output = self.o_proj(attn_output)`
+ * after the attention of LlamaAttention.forward (reference
+ * models/sbvr_llama.py:307-354, the projection at :352) for batch 1, query
+ * length 1.  Same arguments and arithmetic as the attention call, with two
+ * differences.  ctx may be NULL (when given it receives the heads*head_dim
+ * context values the projection consumes).  Both caches are private to this
+ * call and hold their (kv_heads, max_seq, 128) elements in a blocked order, so
+ * that every request of a wave is 1 KiB of consecutive memory: per key/value
+ * head, element (position t, dimension d) lies at
+ *   keys:   (t/16)*2048 + (d/32)*512 + (d%32/8)*128 + (t%16)*8 + d%8
+ *   values: (t/32)*4096 + (d/16)*512 + (t%32/8)*128 + (d%16)*8 + t%8.
+ * Caches that start zero-filled (or whose rows past *pos do not matter) need
+ * no conversion; a cache filled by sbvr_hip_dec_attention_f16 does.
+ * The projection's weight is in the default layout of sbvr_hip_linear_f16 with
+ * K = heads*head_dim: o_bvr (K/32, N, S) uint32, o_coeff_idx (K/G, N) uint8 or
+ * uint16 (idx_bytes), o_coeff_cache (L, S) fp16, o_bias (N) fp16 or NULL (added
+ * after the rounding).
+ * Shapes: head_dim 128, heads = 4 * kv_heads, max_seq a multiple of 32 up to
+ * 4096, N a multiple of 128, S in {2,3,4,6,8}, G a power-of-two multiple of 128;
+ * sbvr_hip_dec_attention_o_supported returns 1 for a shape this call takes, and
+ * anything else gets -2 (run the two calls separately).  Caches, o_bvr and
+ * o_coeff_cache 16-byte aligned.
+ * workspace: sbvr_hip_dec_attention_o_workspace(kv_heads, N) bytes (8 per output
+ * when kv_heads > 1), zero-filled once; every launch leaves it zero-filled, and
+ * launches that share it must not overlap in time (-4 when missing or small).
+ * The result does not depend on the order in which workgroups finish. */
+int sbvr_hip_dec_attention_o_supported(int heads, int kv_heads, int head_dim, int max_seq, int N, int S, int G);
+size_t sbvr_hip_dec_attention_o_workspace(int kv_heads, int N);
+int sbvr_hip_dec_attention_o_f16(const void *qkv, const float *cos_table, const float *sin_table, const float *rot_now,
+                                 const long long *pos, void *kcache, void *vcache, void *ctx, int heads, int kv_heads,
+                                 int head_dim, int max_seq, const uint32_t *o_bvr, const void *o_coeff_idx, int idx_bytes,
+                                 const void *o_coeff_cache, const void *o_bias, void *out, int N, int S, int G, int L,
+                                 void *workspace, size_t workspace_bytes, void *stream);
 
 /* out[ffn] <- fp16(silu(gate)) * up with gate_up = [gate | up] (2*ffn) fp16.
  * Replaces act_fn(gate_proj(x)) * up_proj(x) of LlamaMLP.forward

@@ -56,6 +56,7 @@
 #include <string.h>
 
 #include "../../include/sbvr_hip.h"
+#include "../../include/sbvr_hip_decoder.h"
 
 namespace {
 
@@ -3387,6 +3388,456 @@ sbvr_read_floor_kernel(const v4u *__restrict__ base, uint32_t units, int pattern
 
 } // namespace
 
+namespace {
+
+// ------------------------------------ attention and output projection of one decoded token, one launch
+//
+// The decoder layer's attention (rotary embedding, cache append, softmax(q k^T / sqrt(d)) v over the cached
+// positions; reference models/sbvr_llama.py:193-224, 255-278, 307-354) followed by its SBVR-encoded o_proj, for
+// batch 1 and query length 1, heads of 128 = one sub-group of the projection's K, four query heads per
+// key/value head.  As two launches the pair costs two kernel boundaries and two chains of memory round trips
+// for a few hundred KiB of traffic; here workgroup (g, e) does the attention of key/value head g's four query
+// heads by itself and then multiplies their 512 context values into columns [128 e, 128 e + 128) of the
+// projection, whose K is thereby split kv_heads ways across workgroups (the decode kernel's fixed-point
+// accumulators).  Every workgroup of a key/value head repeats that head's attention (N / 128 times: cheap on the
+// matrix cores, and the head's cache rows come out of one XCD's L2: workgroup i goes to XCD i % 8 and takes
+// head i % kv_heads); nothing waits for another workgroup.
+//   * scores: v_mfma_f32_16x16x32_f16 with 16 cache positions as the rows of A and the four rotated queries as
+//     columns 0..3 of B;
+//   * context: the same instruction with 16 head dimensions as the rows of A and 32 positions as the reduction
+//     index; B holds the softmax weights (fp16, as the reference's fp16 matmul sees them) of the four heads;
+//   * both caches are kept in the element order in which the lanes of those A operands want them, so that
+//     every request of a wave is 1 KiB of consecutive memory.  Per key/value head, element (position t,
+//     dimension d) lies at
+//        keys:   (t/16)*2048 + (d/32)*512 + (d%32/8)*128 + (t%16)*8 + d%8     [block of 16 positions][request j]
+//        values: (t/32)*4096 + (d/16)*512 + (t%32/8)*128 + (d%16)*8 + t%8     [block of 32 positions][16 dimensions]
+//     with lane (col = lane % 16, blk = lane / 16) reading the 8 elements at + blk*128 + col*8;
+//   * a wave asks for things in the order it needs them and no earlier than it must: the new token's q, k, v,
+//     the position and its line indices, then the first 256 positions' keys; after the first barrier the
+//     values and coefficient lines; after the scores the plane words of its two units of the projection (head
+//     wave / 4, columns 32 (wave % 4) .. + 31 of the window).  Rows past the position are fetched for nothing;
+//   * the row of the position itself is never taken from the cache: workgroups with e == 0 append it, the
+//     others (and they) use their own copy;
+//   * the kernel is bound by the instructions its sixteen waves issue, four to a SIMD, not by its MFMAs: work
+//     that only one block of positions needs (the new key, masking of values at and past the position) sits
+//     behind wave-uniform branches, and a head's A operand for the projection is made by one wave, not four.
+// Rounding points are the reference's: rotated q and k, scores, softmax weights and context in fp16; the
+// projection is exact in its activations (three fp8 terms) with one rounding at the end.
+constexpr int kAoWaves = 16, kAoThreads = 64 * kAoWaves;
+constexpr int kAoHead = 128;         // head size
+constexpr int kAoGroup = 4;          // query heads per key/value head
+constexpr int kAoCols = 128;         // output columns of a workgroup: per head 4 waves x 2 column tiles
+constexpr int kAoMaxSeq = 4096;      // 24 bytes of LDS per cache position
+constexpr int kAoLdsFixed = 8192 + kAoWaves * 2048;
+
+struct AttnOArgs {
+    const uint16_t *qkv;          // [heads | kv_heads | kv_heads] x 128 of the new token
+    const float *cos_t, *sin_t;   // (max_seq, 64)
+    const float *rot_now;         // row *pos of cos | sin, or NULL
+    const long long *pos_p;
+    uint16_t *kcache;             // (kv_heads, max_seq * 128), blocked: see the kernel
+    uint16_t *vcache;             // (kv_heads, max_seq * 128), blocked
+    uint16_t *ctx;                // (heads * 128) or NULL
+    int heads, kv_heads, max_seq;
+    // the projection (default layout), K = heads * 128
+    const uint32_t *bvr;
+    const void *idx;
+    const uint16_t *cache;
+    const uint16_t *bias;
+    uint16_t *out;                // (N)
+    unsigned long long *acc;      // (N) split-K accumulators, all zero between calls (kv_heads > 1)
+    int N, L, gshift, idx16;
+};
+
+typedef v4u __attribute__((may_alias)) v4u_alias;      // 16-byte reads of memory written as fp16 elements
+
+#ifdef SBVR_TRACE
+__device__ unsigned long long g_ao_trace[2 * 16 * 12];      // development builds: timestamps of the waves of two workgroups
+#define SBVR_AOSTAMP(i)                                                                                         \
+    do {                                                                                                        \
+        if ((blockIdx.x == 0 || blockIdx.x == 100) && (threadIdx.x & 63) == 0)                                  \
+            g_ao_trace[((blockIdx.x != 0) * 16 + (threadIdx.x >> 6)) * 12 + (i)] = wall_clock64();              \
+    } while (0)
+#else
+#define SBVR_AOSTAMP(i) do { } while (0)
+#endif
+
+template <int S>
+__global__ void __launch_bounds__(kAoThreads)
+sbvr_attn_o_kernel(const AttnOArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int max_seq = a.max_seq;
+    uint16_t *const qn = reinterpret_cast<uint16_t *>(smem);               // rotated queries of the group: 4 x 128
+    uint16_t *const kn = qn + kAoGroup * kAoHead;                          // rotated new key
+    uint16_t *const vn = kn + kAoHead;                                     // new value
+    float *const red_max = reinterpret_cast<float *>(smem + 1536);         // [wave][head]
+    float *const red_sum = red_max + kAoWaves * kAoGroup;                  // [wave]
+    float *const a_scale = red_sum + kAoWaves;                             // [head]: 2^-(e+1) of its A operand
+    float *const part = reinterpret_cast<float *>(smem + 2048);            // [position half][head][dimension]
+    float *const ysum = reinterpret_cast<float *>(smem + 6144);            // [head][column of the window]
+    unsigned char *const abuf = smem + 8192;                               // the heads' A operand images, 2 KiB each
+    float *const scores = reinterpret_cast<float *>(smem + kAoLdsFixed);   // [head][position]
+    uint16_t *const wts = reinterpret_cast<uint16_t *>(scores + kAoGroup * max_seq);   // [head][position], fp16
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 15, blk = lane >> 4;
+    const int g = static_cast<int>(blockIdx.x) % a.kv_heads;       // key/value head
+    const int e = static_cast<int>(blockIdx.x) / a.kv_heads;       // window of the projection's columns
+    const int N = a.N;
+    uint16_t *const kc = a.kcache + static_cast<size_t>(g) * max_seq * kAoHead;
+    uint16_t *const vc = a.vcache + static_cast<size_t>(g) * max_seq * kAoHead;
+    const v4u zero4 = {0u, 0u, 0u, 0u};
+
+    // -- 1. requests that need no position, in the order they are wanted
+    const long long p64 = *a.pos_p;
+    SBVR_AOSTAMP(0);
+    // the new token: waves 0..3 take query head `wave` of the group, wave 4 the key, wave 5 the value; lane d
+    // holds elements d and d + 64 (a rotation pair)
+    uint16_t na = 0, nb = 0;
+    float c_now = 0.f, s_now = 0.f;
+    if (wave < 6) {                          // wave-uniform
+        const int row = wave < 4 ? kAoGroup * g + wave : (wave == 4 ? a.heads + g : a.heads + a.kv_heads + g);
+        const uint16_t *src = a.qkv + static_cast<size_t>(row) * kAoHead;
+        na = src[lane];
+        nb = src[lane + kAoHead / 2];
+        if (wave < 5 && a.rot_now) {
+            c_now = a.rot_now[lane];
+            s_now = a.rot_now[kAoHead / 2 + lane];
+        }
+    }
+    // the projection: head hq = wave / 4 of the group is sub-group sgk of its K; the wave's 32 columns, whose line
+    // indices lane l % 32 asks for
+    const int hq = wave >> 2;
+    const int sgk = kAoGroup * g + hq;
+    const int n0 = e * kAoCols + 32 * (wave & 3);
+    const size_t irow = static_cast<size_t>(sgk >> a.gshift) * N + n0 + (lane & 31);
+    const int lraw = a.idx16 ? static_cast<int>(static_cast<const uint16_t *>(a.idx)[irow])
+                             : static_cast<int>(static_cast<const uint8_t *>(a.idx)[irow]);
+    // keys: wave w takes the 16-position blocks w, w + 16, ...: 2048 elements each, four requests of 1 KiB
+    v4u kpre[4];
+    {
+        const uint16_t *kb = kc + static_cast<size_t>(min(wave, max_seq / 16 - 1)) * 2048 + lane * 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            kpre[j] = *reinterpret_cast<const v4u_alias *>(kb + j * 512);
+    }
+    // (the values and the projection's plane words are asked for further down, each as late as its use allows: a
+    // CU takes about 48 requests of 1 KiB at a time, and a wave that stands in the queue with requests it needs
+    // last keeps all sixteen from their first barrier)
+    __builtin_amdgcn_sched_barrier(0);
+    SBVR_AOSTAMP(1);
+
+    // -- 2. the position is here: rotate, leave q, k, v of the new token in LDS, append (e == 0)
+    const int p = p64 < 0 ? 0 : (p64 >= max_seq ? max_seq - 1 : static_cast<int>(p64));
+    SBVR_AOSTAMP(2);
+    if (wave < 5) {
+        if (!a.rot_now) {
+            c_now = a.cos_t[static_cast<size_t>(p) * (kAoHead / 2) + lane];
+            s_now = a.sin_t[static_cast<size_t>(p) * (kAoHead / 2) + lane];
+        }
+        const float xa = h2f(na), xb = h2f(nb);
+        const uint16_t r0 = f2h(xa * c_now - xb * s_now), r1 = f2h(xb * c_now + xa * s_now);
+        uint16_t *const dst = wave < 4 ? qn + wave * kAoHead : kn;
+        dst[lane] = r0;
+        dst[lane + kAoHead / 2] = r1;
+        if (wave == 4 && e == 0) {
+            // dimension d of position p: block p / 16, request d / 32, lane (d % 32 / 8, p % 16), element d % 8
+            uint16_t *const at = kc + static_cast<size_t>(p >> 4) * 2048 + (lane >> 5) * 512 + ((lane & 31) >> 3) * 128 +
+                                 (p & 15) * 8 + (lane & 7);
+            at[0] = r0;
+            at[1024] = r1;                   // d + 64: two requests on
+        }
+    } else if (wave == 5) {
+        vn[lane] = na;
+        vn[lane + kAoHead / 2] = nb;
+        if (e == 0) {
+            // dimension d of position p: block p / 32, dimensions block d / 16, lane (p % 32 / 8, d % 16), element p % 8
+            uint16_t *const at = vc + static_cast<size_t>(p >> 5) * 4096 + (lane >> 4) * 512 + ((p & 31) >> 3) * 128 +
+                                 (lane & 15) * 8 + (p & 7);
+            at[0] = na;
+            at[2048] = nb;                   // d + 64: four blocks of dimensions on
+        }
+    }
+    __syncthreads();
+    SBVR_AOSTAMP(3);
+    // values: wave (db = w % 8, ph = w / 8) takes dimensions 16 db .. + 15 of the 32-position blocks ph, ph + 2, ...:
+    // 512 elements of each block, one request of 1 KiB
+    const int db = wave & 7, ph = wave >> 3;
+    const uint16_t *const vb = vc + db * 512 + lane * 8;
+    v4u vpre[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        vpre[i] = *reinterpret_cast<const v4u_alias *>(vb + static_cast<size_t>(min(ph + 2 * i, max_seq / 32 - 1)) * 4096);
+    // (the line indices came with the position: lane l gathers the coefficient line of column n0 + l % 32)
+    constexpr int CW = (S + 1) / 2;
+    uint32_t cl[CW];
+    load_line_words<S>(a.cache + static_cast<size_t>(min(lraw, a.L - 1)) * S, cl);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // -- 3. scores of the group's four heads (columns 0..3 of the product; the other columns are not used)
+    const float scaling = rsqrtf(static_cast<float>(kAoHead));
+    v8h qb[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const v4u t = *reinterpret_cast<const v4u_alias *>(qn + (col & (kAoGroup - 1)) * kAoHead + 32 * j + 8 * blk);
+        qb[j] = __builtin_bit_cast(v8h, col < kAoGroup ? t : zero4);
+    }
+    float mx = -INFINITY;                     // of head `col` over the positions this lane sees
+    auto score_block = [&](int tb, v4u (&kw)[4]) __attribute__((always_inline)) {
+        if ((p >> 4) == tb) {                 // wave-uniform: the block of the new key, which is not taken from the cache
+            if (col == (p & 15)) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    kw[j] = *reinterpret_cast<const v4u_alias *>(kn + 32 * j + 8 * blk);
+            }
+        }
+        v4f d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, kw[j]), qb[j], d, 0, 0, 0);
+        // the lane holds head `col`, positions 16 tb + 4 blk + i (the reference's q @ k^T is an fp16 matmul)
+        const int t0 = 16 * tb + 4 * blk;
+        if (col < kAoGroup) {
+            float *const sp = scores + col * max_seq + t0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float v = h2f(f2h(d[i])) * scaling;
+                if (t0 + i <= p) {
+                    sp[i] = v;
+                    mx = fmaxf(mx, v);
+                }
+            }
+        }
+    };
+    if (16 * wave <= p)                       // wave-uniform
+        score_block(wave, kpre);
+    for (int tb = wave + kAoWaves; 16 * tb <= p; tb += kAoWaves) {
+        v4u kw[4];
+        const uint16_t *kb = kc + static_cast<size_t>(tb) * 2048 + lane * 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            kw[j] = *reinterpret_cast<const v4u_alias *>(kb + j * 512);
+        score_block(tb, kw);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    if (lane < kAoGroup)
+        red_max[wave * kAoGroup + lane] = mx;
+    __syncthreads();
+    SBVR_AOSTAMP(4);
+    // the plane words of the wave's two units of the projection
+    Planes<S> q[2];
+    {
+        const uint32_t *wrow = a.bvr + (static_cast<size_t>(4 * sgk + blk) * N + n0 + col) * S;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            q[u] = load_planes<S, true>(wrow + 16 * u * S);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // -- 4. softmax: thread (head hs = tid / 256, slot tid % 256) takes positions slot, slot + 256, ...
+    const int hs = tid >> 8, slot = tid & 255;
+    float *const srow = scores + hs * max_seq;
+    float top = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kAoWaves; ++w)
+        top = fmaxf(top, red_max[w * kAoGroup + hs]);
+    float sum = 0.f;
+    for (int t = slot; t <= p; t += 256) {
+        const float ex = __expf(srow[t] - top);
+        srow[t] = ex;
+        sum += ex;
+    }
+    sum = wave_fsum(sum);
+    if (lane == 0)
+        red_sum[wave] = sum;
+    __syncthreads();
+    const float inv = 1.f / ((red_sum[4 * hs] + red_sum[4 * hs + 1]) + (red_sum[4 * hs + 2] + red_sum[4 * hs + 3]));
+    const int t_pad = (p + 32) & ~31;         // the context products go over whole blocks of 32 positions
+    for (int t = slot; t < t_pad; t += 256)   // (weights are rounded to fp16; positions past p weigh nothing)
+        wts[hs * max_seq + t] = t <= p ? f2h(srow[t] * inv) : static_cast<uint16_t>(0);
+    __syncthreads();
+    SBVR_AOSTAMP(5);
+
+    // -- 5. context: dimensions 16 db .. + 15 over the wave's blocks of 32 positions
+    v4f o = {0.f, 0.f, 0.f, 0.f};
+    const uint16_t *const wrow_l = wts + (col & (kAoGroup - 1)) * max_seq + 8 * blk;
+    auto context_block = [&](int pb, v4u vw) __attribute__((always_inline)) {
+        if (32 * pb + 31 >= p) {              // wave-uniform: the block of p (later blocks are not visited)
+            // positions before p come from the cache, p itself from the new token, later ones may hold anything
+            const int ts = 32 * pb + 8 * blk;     // the lane's positions ts .. ts + 7 of dimension 16 db + col
+            const uint32_t vfresh = vn[16 * db + col];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int t_lo = ts + 2 * c, t_hi = t_lo + 1;
+                const uint32_t lo = t_lo < p ? (vw[c] & 0xffffu) : (t_lo == p ? vfresh : 0u);
+                const uint32_t hi = t_hi < p ? (vw[c] >> 16) : (t_hi == p ? vfresh : 0u);
+                vw[c] = lo | (hi << 16);
+            }
+        }
+        const v4u wb = *reinterpret_cast<const v4u_alias *>(wrow_l + 32 * pb);
+        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, vw),
+                                                   __builtin_bit_cast(v8h, col < kAoGroup ? wb : zero4), o, 0, 0, 0);
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (32 * (ph + 2 * i) <= p)           // wave-uniform
+            context_block(ph + 2 * i, vpre[i]);
+    for (int pb = ph + 8; 32 * pb <= p; pb += 2)
+        context_block(pb, *reinterpret_cast<const v4u_alias *>(vb + static_cast<size_t>(pb) * 4096));
+    // the lane holds head `col`, dimensions 16 db + 4 blk + i
+    if (col < kAoGroup)
+        *reinterpret_cast<v4f *>(part + (ph * kAoGroup + col) * kAoHead + 16 * db + 4 * blk) = o;
+    __syncthreads();
+    SBVR_AOSTAMP(6);
+
+    // -- 6. a head's context row as the one batch row of the projection's A operand (the decode kernel's step 2:
+    //       three fp8 terms per element, written where the MFMA wants them through 2 KiB of LDS); made once per
+    //       head, by waves 0, 5, 10 and 15 (one on each SIMD)
+    if (wave == 5 * hq) {                     // wave-uniform
+        const float2 c0 = reinterpret_cast<const float2 *>(part + hq * kAoHead)[lane];
+        const float2 c1 = reinterpret_cast<const float2 *>(part + (kAoGroup + hq) * kAoHead)[lane];
+        const uint32_t v = static_cast<uint32_t>(f2h(c0.x + c1.x)) | (static_cast<uint32_t>(f2h(c0.y + c1.y)) << 16);
+        if (a.ctx && e == 0)
+            reinterpret_cast<uint32_t *>(a.ctx + static_cast<size_t>(sgk) * kAoHead)[lane] = v;
+        unsigned char *const mine = abuf + hq * 2048;
+        reinterpret_cast<uint4 *>(mine)[lane * 2] = uint4{0u, 0u, 0u, 0u};
+        reinterpret_cast<uint4 *>(mine)[lane * 2 + 1] = uint4{0u, 0u, 0u, 0u};
+        const uint32_t amax = wave_umax(max(v & 0x7fffu, (v >> 16) & 0x7fffu));
+        const int eh = min(max(static_cast<int>(amax >> 10), 1), 30);
+        const int ex2 = 20 - eh;              // 2^ex2 puts the head's largest magnitude into [32, 64)
+        if (lane == 0)
+            a_scale[hq] = __uint_as_float(static_cast<uint32_t>(126 - ex2) << 23);
+        const int off = a_image_byte_offset(8 * (lane >> 2) + (lane & 3), 0);
+        const uint32_t half_sel = (lane & 1) ? 0x07060302u : 0x05040100u;
+        const int fac_log2 = (lane & 3) == 0 ? 2 : ((lane & 3) == 1 ? 1 : 0);
+        const int va = __builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x50, 0xF, 0xF, true);   // quad_perm 0,0,1,1
+        const int vb2 = __builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xFA, 0xF, 0xF, true);  // quad_perm 2,2,3,3
+        v2h z = as_v2h(__builtin_amdgcn_perm(static_cast<uint32_t>(vb2), static_cast<uint32_t>(va), half_sel));
+        const float sc = __uint_as_float(static_cast<uint32_t>(127 - ex2 - fac_log2) << 23);
+        const float sc_last = __uint_as_float(static_cast<uint32_t>(127 - 8 - ex2 - fac_log2) << 23);
+        v2s b = {0, 0};
+        b = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(b, z, sc, false);
+        z -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(as_int(b), sc, false);
+        b = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(b, z, sc, true);
+        z -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(as_int(b), sc, true);
+        const v2s b3 = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(v2s{0, 0}, z, sc_last, false);
+        *reinterpret_cast<short *>(mine + off + 0 * 32) = b[0];
+        *reinterpret_cast<short *>(mine + off + 1 * 32) = b[1];
+        *reinterpret_cast<short *>(mine + off + 2 * 32) = b3[0];
+    }
+    __syncthreads();
+    const v8i A = *reinterpret_cast<const v8i *>(abuf + hq * 2048 + lane * 32);
+    const float scale = a_scale[hq];
+    SBVR_AOSTAMP(7);
+
+    // -- 7. the wave's two units: plane sums, coefficients (lane 16 u + col gathered the line of this lane's column)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        float ps[S];
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            const uint32_t w = q[u].w[j];
+            v8i B;
+            B[0] = static_cast<int>(w & 0x11111111u);
+            B[1] = static_cast<int>(w & 0x22222222u);
+            B[2] = static_cast<int>(w & 0x44444444u);
+            B[3] = static_cast<int>((w >> 1) & 0x44444444u);
+            B[4] = 0; B[5] = 0; B[6] = 0; B[7] = 0;
+            const v4f zf = {0.f, 0.f, 0.f, 0.f};
+            const v4f d = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, zf, 0, 4, 0, 0, 0, 0);
+            ps[j] = fmaf(d[2], 1.f / kLastTermScale, d[0] + d[1]);
+        }
+        uint32_t cw[CW];
+#pragma unroll
+        for (int j = 0; j < CW; ++j)
+            cw[j] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute((16 * u + col) * 4, static_cast<int>(cl[j])));
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < S; ++j)
+            acc = fmaf(h2f(static_cast<uint16_t>(j & 1 ? cw[j / 2] >> 16 : cw[j / 2] & 0xffffu)), ps[j], acc);
+        if (blk == 0)                         // (rows 0..2 of the product are the three terms of the one batch row)
+            ysum[hq * kAoCols + 32 * (wave & 3) + 16 * u + col] = acc * scale;
+    }
+    __syncthreads();
+    SBVR_AOSTAMP(8);
+
+    // -- 8. the four heads' partial results added in a fixed order; K is split kv_heads ways across workgroups
+    if (tid < kAoCols) {
+        float total = (ysum[tid] + ysum[kAoCols + tid]) + (ysum[2 * kAoCols + tid] + ysum[3 * kAoCols + tid]);
+        const int n = e * kAoCols + tid;
+        bool last = true;
+        if (a.kv_heads > 1) {
+            unsigned long long tot = (1ull << 56) + static_cast<unsigned long long>(to_fixed(total) + kAccBias);
+            tot += __hip_atomic_fetch_add(a.acc + n, tot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last = static_cast<int>(tot >> 56) == a.kv_heads;
+            if (last) {
+                const long long sum56 = static_cast<long long>(tot & ((1ull << 56) - 1)) - (static_cast<long long>(a.kv_heads) << 47);
+                const float hi = static_cast<float>(static_cast<int>(sum56 >> 24));
+                const float lo = static_cast<float>(static_cast<int>(sum56 & 0xffffff));
+                total = fmaf(hi, 1.f / (1 << (kAccFracBits - 24)), lo * (1.f / (1 << kAccFracBits)));
+                __hip_atomic_store(a.acc + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (last) {
+            uint16_t r = f2h(total);
+            if (a.bias)
+                r = hadd(r, a.bias[n]);
+            a.out[n] = r;
+        }
+    }
+    SBVR_AOSTAMP(9);
+}
+
+template <int S>
+hipError_t launch_attn_o_inst(const AttnOArgs &a, hipStream_t st)
+{
+    const dim3 grid(static_cast<unsigned>(a.kv_heads * (a.N / kAoCols))), block(kAoThreads);
+    const size_t lds = kAoLdsFixed + 24 * static_cast<size_t>(a.max_seq);
+    if (lds > 65536) {          // above what a kernel gets without asking
+        static bool raised_on[16] = {};
+        std::lock_guard<std::mutex> guard(g_dev_lock);
+        int dev_now = 0;
+        if (hipGetDevice(&dev_now) != hipSuccess || dev_now < 0 || dev_now >= 16)
+            dev_now = 0;
+        if (!raised_on[dev_now]) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sbvr_attn_o_kernel<S>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess)
+                return e;
+            raised_on[dev_now] = true;
+        }
+    }
+    hipLaunchKernelGGL((sbvr_attn_o_kernel<S>), grid, block, lds, st, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_attn_o(int S, const AttnOArgs &a, hipStream_t st)
+{
+    switch (S) {
+    case 4: return launch_attn_o_inst<4>(a, st);
+#ifndef SBVR_FAST_BUILD
+    case 2: return launch_attn_o_inst<2>(a, st);
+    case 3: return launch_attn_o_inst<3>(a, st);
+    case 6: return launch_attn_o_inst<6>(a, st);
+    case 8: return launch_attn_o_inst<8>(a, st);
+#endif
+    default: return hipErrorInvalidConfiguration;
+    }
+}
+
+bool attn_o_shape_ok(int heads, int kv_heads, int head_dim, int max_seq, int N, int S, int G)
+{
+    return kv_heads >= 1 && kv_heads <= kMaxKsplit && heads == kAoGroup * kv_heads && head_dim == kAoHead &&
+           max_seq >= 32 && max_seq <= kAoMaxSeq && max_seq % 32 == 0 && N >= kAoCols && N % kAoCols == 0 &&
+           mfma_path_ok(1, N, heads * kAoHead, S, G);
+}
+
+} // namespace
+
 // Scratch memory of sbvr_hip_linear_f16_noalloc: the split-K accumulators of the decode kernel, for callers
 // that cannot bring a workspace.  One copy per GPU the library runs on, held until the process ends; zero when
 // the module is loaded, and every launch leaves it zero (the adder that completes an accumulator resets it).
@@ -3428,9 +3879,13 @@ extern "C" {
 
 #ifdef SBVR_TRACE
 void sbvr_hip_debug_set_trace(unsigned long long *p) { g_trace = p; }
+int sbvr_hip_debug_attn_o_trace(unsigned long long *out384)
+{
+    return hipMemcpyFromSymbol(out384, HIP_SYMBOL(g_ao_trace), sizeof(g_ao_trace)) == hipSuccess ? 0 : -3;
+}
 #endif
 
-int sbvr_hip_version(void) { return 103; }      // 101: the one-row linears with a fused prologue; 102: _noalloc, _stream_floor; 103: _read_floor
+int sbvr_hip_version(void) { return 104; }      // 101: the one-row linears with a fused prologue; 102: _noalloc, _stream_floor; 103: _read_floor; 104: _dec_attention_o
 
 const char *sbvr_hip_last_error(void) { return g_err; }
 
@@ -4056,6 +4511,75 @@ int sbvr_hip_mm_T_ws(const uint32_t *l_bvr, const void *l_coeff_idx, int l_idx_b
     return SBVR_HIP_OK;
 }
 
+
+int sbvr_hip_dec_attention_o_supported(int heads, int kv_heads, int head_dim, int max_seq, int N, int S, int G)
+{
+    if (S != 2 && S != 3 && S != 4 && S != 6 && S != 8)
+        return 0;
+#ifdef SBVR_FAST_BUILD
+    if (S != 4)
+        return 0;
+#endif
+    return attn_o_shape_ok(heads, kv_heads, head_dim, max_seq, N, S, G) ? 1 : 0;
+}
+
+size_t sbvr_hip_dec_attention_o_workspace(int kv_heads, int N)
+{
+    return kv_heads > 1 && N > 0 ? static_cast<size_t>(N) * sizeof(unsigned long long) : 0;
+}
+
+int sbvr_hip_dec_attention_o_f16(const void *qkv, const float *cos_table, const float *sin_table, const float *rot_now,
+                                 const long long *pos, void *kcache, void *vcache, void *ctx, int heads, int kv_heads,
+                                 int head_dim, int max_seq, const uint32_t *o_bvr, const void *o_coeff_idx, int idx_bytes,
+                                 const void *o_coeff_cache, const void *o_bias, void *out, int N, int S, int G, int L,
+                                 void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!qkv || !cos_table || !sin_table || !pos || !kcache || !vcache || !o_bvr || !o_coeff_idx || !o_coeff_cache || !out)
+        return fail(SBVR_HIP_EINVAL, "null pointer argument");
+    if (heads <= 0 || kv_heads <= 0 || head_dim <= 0 || max_seq <= 0 || N <= 0 || S <= 0 || G <= 0 || L <= 0)
+        return fail(SBVR_HIP_EINVAL, "non-positive size");
+    if (idx_bytes != 1 && idx_bytes != 2)
+        return fail(SBVR_HIP_EINVAL, "idx_bytes must be 1 or 2, got %d", idx_bytes);
+    if (idx_bytes == 1 && L > 256)
+        return fail(SBVR_HIP_EINVAL, "uint8 indices cannot address L=%d lines", L);
+    if (!sbvr_hip_dec_attention_o_supported(heads, kv_heads, head_dim, max_seq, N, S, G))
+        return fail(SBVR_HIP_EUNSUPPORTED, "attention + projection in one launch: heads=%d kv_heads=%d head_dim=%d max_seq=%d N=%d S=%d G=%d",
+                    heads, kv_heads, head_dim, max_seq, N, S, G);
+    if ((reinterpret_cast<uintptr_t>(kcache) | reinterpret_cast<uintptr_t>(vcache) | reinterpret_cast<uintptr_t>(o_bvr) |
+         reinterpret_cast<uintptr_t>(o_coeff_cache)) % 16 ||
+        (reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(o_coeff_idx)) % 2 ||
+        (ctx && reinterpret_cast<uintptr_t>(ctx) % 4))
+        return fail(SBVR_HIP_EINVAL, "caches, bvr and coeff_cache must be 16-byte aligned, ctx 4-byte, qkv, out and uint16 indices 2-byte");
+    if (kv_heads > 1 && (!workspace || workspace_bytes < sbvr_hip_dec_attention_o_workspace(kv_heads, N) ||
+                         reinterpret_cast<uintptr_t>(workspace) % 8 != 0))
+        return fail(SBVR_HIP_EWORKSPACE, "attention + projection needs %zu bytes of zeroed workspace (8-byte aligned), got %zu",
+                    sbvr_hip_dec_attention_o_workspace(kv_heads, N), workspace_bytes);
+    AttnOArgs a{};
+    a.qkv = static_cast<const uint16_t *>(qkv);
+    a.cos_t = cos_table;
+    a.sin_t = sin_table;
+    a.rot_now = rot_now;
+    a.pos_p = pos;
+    a.kcache = static_cast<uint16_t *>(kcache);
+    a.vcache = static_cast<uint16_t *>(vcache);
+    a.ctx = static_cast<uint16_t *>(ctx);
+    a.heads = heads; a.kv_heads = kv_heads; a.max_seq = max_seq;
+    a.bvr = o_bvr;
+    a.idx = o_coeff_idx;
+    a.cache = static_cast<const uint16_t *>(o_coeff_cache);
+    a.bias = static_cast<const uint16_t *>(o_bias);
+    a.out = static_cast<uint16_t *>(out);
+    a.acc = static_cast<unsigned long long *>(workspace);
+    a.N = N; a.L = L;
+    a.gshift = __builtin_ctz(static_cast<unsigned>(G / kSub));
+    a.idx16 = idx_bytes == 2;
+    const hipError_t e = launch_attn_o(S, a, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess)
+        return fail(SBVR_HIP_ELAUNCH, "attention + projection launch: %s", hipGetErrorString(e));
+    g_last_kernel = SBVR_HIP_KERNEL_DECODE;
+    g_last_rounding = SBVR_HIP_ROUNDING_EXACT;
+    return SBVR_HIP_OK;
+}
 
 int sbvr_hip_read_floor(const void *buf, size_t buf_bytes, size_t bytes, int workgroups, int waves, int ahead, int pattern,
                         int row_bytes, int win_bytes, void *sink, void *stream)

@@ -71,11 +71,18 @@ class _Linear:
 
 class SbvrLlamaDecoder:
     def __init__(self, shape=None, device="cuda:0", num_sums=4, bvr_len=128, lines=256, max_seq=256, seed=0,
-                 fused=True):
+                 fused=True, attention_o=None):
         self.shape = s = shape or LlamaShape()
         # fused: the residual add + norm and the SiLU * up run inside the linear that follows them
         # (5 launches per layer instead of 8)
         self.fused = fused
+        # attention_o: attention and the o projection in one launch (4 launches per layer) where the shape has
+        # that kernel; None = wherever it has.  The caches are then kept in that kernel's blocked element order.
+        supported = fused and hip.dec_attention_o_supported(s.heads, s.kv_heads, s.head_dim, max_seq, s.hidden,
+                                                            num_sums, bvr_len)
+        if attention_o and not supported:
+            raise ValueError("attention_o: this shape has no fused attention + projection kernel")
+        self.attention_o = supported if attention_o is None else bool(attention_o)
         self.device = dev = torch.device(device)
         self.max_seq = max_seq
         hip._sbvr_hip_init(dev)
@@ -158,7 +165,8 @@ class SbvrLlamaDecoder:
     def _step_fused(self):
         """One launch for the end of the step (final norm, head, argmax) where the
         hidden size has a kernel, and 5 launches per layer: q|k|v (with the residual add and norm in front),
-        attention, o, gate|up (same), down (with SiLU*up in front).  The residual
+        attention, o, gate|up (same), down (with SiLU*up in front); 4 with attention and o in one launch
+        (self.attention_o).  The residual
         stream alternates between two buffers: a linear reads one and writes the
         sum to the other, since its workgroups do not run in step."""
         s = self.shape
@@ -169,9 +177,15 @@ class SbvrLlamaDecoder:
             qkv = layer["qkv"].after_add_rmsnorm(a, delta, layer["norm1"], s.rms_eps, b)
             if self.probe is not None:
                 self.probe(number, b)
-            hip.dec_attention(qkv, self.cos, self.sin, self.pos, layer["k"], layer["v"], ctx,
-                              s.heads, s.kv_heads, s.head_dim, self.rot_now)
-            delta = layer["o"](ctx)
+            if self.attention_o:
+                o = layer["o"]
+                delta = hip.dec_attention_o(qkv, self.cos, self.sin, self.pos, layer["k"], layer["v"], s.heads,
+                                            s.kv_heads, s.head_dim, o.bvr, o.idx, o.cache, None, o.bvr_len,
+                                            out=o.out, rot_now=self.rot_now)
+            else:
+                hip.dec_attention(qkv, self.cos, self.sin, self.pos, layer["k"], layer["v"], ctx,
+                                  s.heads, s.kv_heads, s.head_dim, self.rot_now)
+                delta = layer["o"](ctx)
             gate_up = layer["gate_up"].after_add_rmsnorm(b, delta, layer["norm2"], s.rms_eps, a)
             delta = layer["down"].after_swiglu(gate_up)
         if self.probe is not None:

@@ -66,6 +66,11 @@ def _load():
     fp = ctypes.POINTER(ctypes.c_float)
     lib.sbvr_hip_dec_add_rmsnorm_f16.argtypes = [vp, vp, vp, vp, i, ctypes.c_float, vp]
     lib.sbvr_hip_dec_attention_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
+    lib.sbvr_hip_dec_attention_o_supported.argtypes = [i, i, i, i, i, i, i]
+    lib.sbvr_hip_dec_attention_o_workspace.restype = sz
+    lib.sbvr_hip_dec_attention_o_workspace.argtypes = [i, i]
+    lib.sbvr_hip_dec_attention_o_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, i, vp, vp, vp,
+                                                 i, i, i, i, vp, sz, vp]
     lib.sbvr_hip_dec_silu_mul_f16.argtypes = [vp, vp, i, vp]
     lib.sbvr_hip_dec_argmax_advance_f16.argtypes = [vp, i, vp, vp, vp, i, vp, vp, i, vp, vp]
     lib.sbvr_hip_dec_head_argmax_f16.argtypes = [vp, vp, vp, ctypes.c_float, vp, i, i, vp, vp, vp, vp, i, vp, vp, i,
@@ -378,6 +383,79 @@ def dec_attention(qkv, cos, sin, pos, kcache, vcache, ctx, heads, kv_heads, head
                                                    ctx.data_ptr(), heads, kv_heads, head_dim, max_seq, _stream()),
                "attention")
     return ctx
+
+
+def dec_attention_o_supported(heads, kv_heads, head_dim, max_seq, N, S, G):
+    """Whether ``dec_attention_o`` takes this shape (else: ``dec_attention``, then the linear)."""
+    return bool(_load().sbvr_hip_dec_attention_o_supported(heads, kv_heads, head_dim, max_seq, N, S, G))
+
+
+def attention_o_cache_layout(cache, inverse=False, values=False):
+    """(kv_heads, max_seq, 128) fp16 in the natural order -> the blocked order ``dec_attention_o`` keeps its caches
+    in (same shape, other element order), or back with ``inverse``.  Keys: blocks of 16 positions, each as four
+    runs (dimensions 32 j .. 32 j + 31) of [dimension % 32 // 8][position % 16][dimension % 8].  Values: blocks of
+    32 positions, each as eight runs (dimensions 16 b .. 16 b + 15) of [position % 32 // 8][dimension % 16][position % 8]."""
+    kv, T, D = cache.shape
+    if D != 128 or T % 32:
+        raise ValueError("attention_o_cache_layout: head_dim 128 and max_seq a multiple of 32")
+    if not values:
+        if not inverse:       # (tb, col, j, blk, i) -> (tb, j, blk, col, i)
+            return cache.view(kv, T // 16, 16, 4, 4, 8).permute(0, 1, 3, 4, 2, 5).contiguous().view(kv, T, D)
+        return cache.view(kv, T // 16, 4, 4, 16, 8).permute(0, 1, 4, 2, 3, 5).contiguous().view(kv, T, D)
+    if not inverse:           # (pb, blk, i, db, col) -> (pb, db, blk, col, i)
+        return cache.view(kv, T // 32, 4, 8, 8, 16).permute(0, 1, 4, 2, 5, 3).contiguous().view(kv, T, D)
+    return cache.view(kv, T // 32, 8, 4, 16, 8).permute(0, 1, 3, 5, 2, 4).contiguous().view(kv, T, D)
+
+
+def dec_attention_o(qkv, cos, sin, pos, kcache, vcache, heads, kv_heads, head_dim, bvr, coeff_idx, coeff_cache,
+                    bias=None, bvr_len=None, out=None, rot_now=None, ctx=None):
+    """``dec_attention`` and the encoded output projection of its context row in one launch.  Both caches are
+    (kv_heads, max_seq, head_dim) fp16 in the blocked element order of ``attention_o_cache_layout``.  ``ctx``
+    (heads * head_dim fp16), when given, receives the context row.  Returns ``out`` (1, N)."""
+    lib = _load()
+    dev = qkv.device
+    for t, name in ((qkv, "qkv"), (kcache, "kcache"), (vcache, "vcache")) + (((ctx, "ctx"),) if ctx is not None else ()):
+        _want(t, name, torch.float16, None, dev)
+    _want(cos, "cos", torch.float32, None, dev)
+    _want(sin, "sin", torch.float32, None, dev)
+    _want(pos, "pos", torch.int64, None, dev)
+    max_seq = kcache.shape[1]
+    if kcache.shape != (kv_heads, max_seq, head_dim) or vcache.shape != kcache.shape or \
+            cos.shape != (max_seq, head_dim // 2) or sin.shape != cos.shape or \
+            qkv.numel() != (heads + 2 * kv_heads) * head_dim or (ctx is not None and ctx.numel() != heads * head_dim):
+        raise SbvrHipError("dec_attention_o: tensor shapes do not match heads/kv_heads/head_dim/max_seq")
+    if rot_now is not None:
+        _want(rot_now, "rot_now", torch.float32, None, dev)
+        if rot_now.numel() != head_dim:
+            raise SbvrHipError("dec_attention_o: rot_now must hold head_dim floats")
+    K = heads * head_dim
+    _want(bvr, "bvr", torch.uint32, 3, dev)
+    _want(coeff_idx, "coeff_idx", (torch.uint8, torch.uint16), 2, dev)
+    _want(coeff_cache, "coeff_cache", torch.float16, 2, dev)
+    Kw, N, S = bvr.shape
+    L = coeff_cache.shape[0]
+    if Kw * 32 != K or coeff_idx.shape[1] != N or coeff_cache.shape[1] != S:
+        raise ValueError("the projection's bvr / coeff_idx / coeff_cache do not match heads * head_dim")
+    G = bvr_len if bvr_len is not None else K // coeff_idx.shape[0]
+    if G * coeff_idx.shape[0] != K:
+        raise ValueError(f"coeff_idx has {coeff_idx.shape[0]} groups, K={K}, bvr_len={G}")
+    ib = _idx_bytes(coeff_idx, L, "coeff_idx")
+    if out is None:
+        out = torch.empty((1, N), dtype=torch.float16, device=dev)
+    else:
+        _want(out, "out", torch.float16, 2, dev)
+        if tuple(out.shape) != (1, N):
+            raise ValueError("out has the wrong shape")
+    with torch.cuda.device(dev):
+        need = lib.sbvr_hip_dec_attention_o_workspace(kv_heads, N)
+        ws = _workspace(need, dev) if need else None
+        _check(lib.sbvr_hip_dec_attention_o_f16(
+            qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), rot_now.data_ptr() if rot_now is not None else None,
+            pos.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), ctx.data_ptr() if ctx is not None else None,
+            heads, kv_heads, head_dim, max_seq, bvr.data_ptr(), coeff_idx.data_ptr(), ib, coeff_cache.data_ptr(),
+            _bias_ptr(bias, N, dev), out.data_ptr(), N, S, G, L,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream()))
+    return out
 
 
 def dec_silu_mul(gate_up, out):

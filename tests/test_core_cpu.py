@@ -166,7 +166,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in sbvr_hip.h but not exported"
     lib.sbvr_hip_version.restype = ctypes.c_int
-    assert lib.sbvr_hip_version() == 103
+    assert lib.sbvr_hip_version() == 104
     lib.sbvr_hip_linear_f16_workspace.restype = ctypes.c_size_t
     assert lib.sbvr_hip_linear_f16_workspace(1, 14336, 4096, 4, 128) == 14336 * 8
     assert lib.sbvr_hip_linear_f16_workspace(1, 64, 96, 4, 32) == 0        # portable kernel: no workspace
@@ -260,3 +260,20 @@ def test_fuse_rows_decodes_to_the_stacked_weights(oracle):
     assert small[1].dtype == torch.uint8 and small[2].shape[0] == 200
     with pytest.raises(ValueError):
         layout.fuse_rows([parts[0], synth.random_encoding(16, 512, 3, 128, 10, seed=1)])
+
+
+def test_attention_o_cache_layout_round_trip():
+    """The blocked element order of the one-launch attention + projection's caches (host-side helper): a
+    permutation, its inverse, and the offsets the kernel computes for one element."""
+    import torch
+    from sbvr import hip
+    x = torch.arange(2 * 96 * 128, dtype=torch.float32).view(2, 96, 128)
+    for values in (False, True):
+        y = hip.attention_o_cache_layout(x, values=values)
+        assert y.shape == x.shape and torch.equal(hip.attention_o_cache_layout(y, inverse=True, values=values), x)
+        for t, d in ((0, 0), (37, 77), (95, 127), (16, 32), (31, 8)):
+            if values:
+                off = (t // 32) * 4096 + (d // 16) * 512 + ((t % 32) // 8) * 128 + (d % 16) * 8 + t % 8
+            else:
+                off = (t // 16) * 2048 + (d // 32) * 512 + ((d % 32) // 8) * 128 + (t % 16) * 8 + d % 8
+            assert y[1].flatten()[off] == x[1, t, d]

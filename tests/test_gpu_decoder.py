@@ -110,7 +110,7 @@ def test_full_width_decoder_matches_dense(oracle):
     from sbvr.decoder import LlamaShape, SbvrLlamaDecoder
 
     shape = LlamaShape(layers=2)
-    dec = SbvrLlamaDecoder(shape, "cuda:0", num_sums=4, bvr_len=128, lines=256, max_seq=16, seed=11)
+    dec = SbvrLlamaDecoder(shape, "cuda:0", num_sums=4, bvr_len=128, lines=256, max_seq=32, seed=11)
     for layer in dec.layers:
         for k in ("qkv", "o", "gate_up", "down"):
             layer[k].cache.mul_(1.5)        # (so that the layers move the residual stream; see the small test)
@@ -334,7 +334,7 @@ def test_decoder_with_fused_head(oracle):
     from sbvr.decoder import LlamaShape, SbvrLlamaDecoder
 
     shape = LlamaShape(hidden=512, layers=2, heads=8, kv_heads=2, head_dim=64, ffn=1024, vocab=777)
-    dec = SbvrLlamaDecoder(shape, "cuda:0", lines=64, max_seq=16, seed=11)
+    dec = SbvrLlamaDecoder(shape, "cuda:0", lines=64, max_seq=32, seed=11)
     for layer in dec.layers:
         for k in ("qkv", "o", "gate_up", "down"):
             layer[k].cache.mul_(2.0)
