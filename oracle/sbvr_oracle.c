@@ -213,6 +213,8 @@ void sbvr_oracle_linear_f16(const uint16_t *x, const void *bvr, int word_bits,
                             int mode, uint16_t *y, double *yd)
 {
     int64_t Kg = K / G;
+    /* (every output is one thread's own sequential sum: the threads change nothing in the results) */
+#pragma omp parallel for collapse(2) schedule(static) if (M * N * K > (1 << 22))
     for (int64_t m = 0; m < M; ++m)
         for (int64_t n = 0; n < N; ++n) {
             double acc = 0.0;
