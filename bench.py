@@ -229,6 +229,56 @@ def decode_breakdown(dec):
     return out
 
 
+def attention_o_leg(eager=0):
+    """The decoder layer's attention and o projection at the Llama-3-8B shape (32 / 8 heads of 128, hidden 4096,
+    cache of 256 positions, SBVR S=4 G=128 projection), as one launch (sbvr_hip_dec_attention_o_f16) and as two
+    (sbvr_hip_dec_attention_f16, then the linear), 32 layers' worth of distinct weights and caches replayed from
+    one HIP graph, at three positions.  eager > 0: only that many eager launches of the one-launch form per
+    position (no graph, no timing): what a counter pass of a profiler wants."""
+    import torch
+    from sbvr import hip, synth
+    dev = torch.device("cuda:0")
+    hip._sbvr_hip_init(dev)
+    heads, kv_heads, hd, max_seq, hidden, layers = 32, 8, 128, 256, 4096, 32
+    gen = torch.Generator(device=dev).manual_seed(0)
+    ws = []
+    for l in range(layers):
+        b, i, c = (t.to(dev) for t in synth.random_encoding(hidden, heads * hd, NUM_SUMS, GROUP, LINES, seed=l))
+        kc = torch.randn((kv_heads, max_seq, hd), generator=gen, device=dev).to(torch.float16)
+        vc = torch.randn((kv_heads, max_seq, hd), generator=gen, device=dev).to(torch.float16)
+        ws.append((b, i, c, kc, vc, kc.clone(), vc.clone()))
+    qkv = torch.randn((1, (heads + 2 * kv_heads) * hd), generator=gen, device=dev).to(torch.float16)
+    ang = torch.rand((max_seq, hd // 2), generator=gen, device=dev) * 6.28
+    cos, sin = torch.cos(ang), torch.sin(ang)
+    ctx = torch.empty((1, heads * hd), dtype=torch.float16, device=dev)
+    out = torch.empty((1, hidden), dtype=torch.float16, device=dev)
+    rows = []
+    for p in (128, 200, 255):
+        pos = torch.tensor([p], device=dev)
+        rot = torch.cat((cos[p], sin[p])).contiguous()
+
+        def one(_):
+            for (b, i, c, kc, vc, kb, vb) in ws:
+                hip.dec_attention_o(qkv, cos, sin, pos, kb, vb, heads, kv_heads, hd, b, i, c, None, GROUP, out=out,
+                                    rot_now=rot)
+
+        def two(_):
+            for (b, i, c, kc, vc, kb, vb) in ws:
+                hip.dec_attention(qkv, cos, sin, pos, kc, vc, ctx, heads, kv_heads, hd, rot)
+                hip._sbvr_linear_f16(ctx, b, i, c, None, GROUP, out=out)
+
+        if eager:
+            for _ in range(max(1, eager // layers)):
+                one(0)
+            torch.cuda.synchronize()
+            rows.append({"position": p, "eager_launches": max(1, eager // layers) * layers})
+            continue
+        rows.append({"position": p,
+                     "one_launch_us": round(_graph_time(one, 1) * 1e6 / layers, 2),
+                     "two_launches_us": round(_graph_time(two, 1) * 1e6 / layers, 2)})
+    return rows
+
+
 def _graph_time(fn, iters, stream=None):
     """Seconds per call of fn(i), i = 0..iters-1, recorded into one HIP graph and replayed (best of 3)."""
     import torch
@@ -539,6 +589,11 @@ def main():
     ap.add_argument("--prefill", action="store_true", help="run only the prefill GEMM sizes and print them")
     ap.add_argument("--other-ops", action="store_true",
                     help="run only _sbvr_mm_T and _sbvr_row_deq_mm_T at the layer shapes and print them")
+    ap.add_argument("--attention-o", action="store_true",
+                    help="run only the decoder's attention + o projection, as one launch and as two, and print both")
+    ap.add_argument("--eager", type=int, default=0, metavar="N",
+                    help="with --attention-o: N eager launches of the one-launch form per position instead of timed "
+                         "graph replays (for counter passes of a profiler)")
     ap.add_argument("--stream-floor", action="store_true",
                     help="run only the launch that makes the gate GEMV's memory requests and nothing else "
                          "(sbvr_hip_linear_f16_stream_floor) and print its time beside the kernel's")
@@ -568,6 +623,10 @@ def main():
         return
     if a.read_floor:
         print(json.dumps({"metric": "read-only launches of the gate shape's plane words, us and GB/s", "read_floor": read_floor_leg()}))
+        return
+    if a.attention_o:
+        print(json.dumps({"metric": "decoder attention + SBVR o projection at the 8B shape, us per layer",
+                          "attention_o": attention_o_leg(a.eager)}))
         return
     if a.other_ops:
         print(json.dumps({"metric": "SBVR operator forms of the reference, us and GB/s of algorithmic bytes",
