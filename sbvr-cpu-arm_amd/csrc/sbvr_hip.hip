@@ -3400,8 +3400,8 @@ namespace {
 // heads by itself and then multiplies their 512 context values into columns [128 e, 128 e + 128) of the
 // projection, whose K is thereby split kv_heads ways across workgroups (the decode kernel's fixed-point
 // accumulators).  Every workgroup of a key/value head repeats that head's attention (N / 128 times: cheap on the
-// matrix cores, and the head's cache rows come out of one XCD's L2: workgroup i goes to XCD i % 8 and takes
-// head i % kv_heads); nothing waits for another workgroup.
+// matrix cores, and the head's cache rows come out of one XCD's L2: workgroup (g, e) is number g + kv_heads * e
+// of the launch and workgroups go to the 8 XCDs in turn); nothing waits for another workgroup.
 //   * scores: v_mfma_f32_16x16x32_f16 with 16 cache positions as the rows of A and the four rotated queries as
 //     columns 0..3 of B;
 //   * context: the same instruction with 16 head dimensions as the rows of A and 32 positions as the reduction
@@ -3455,8 +3455,8 @@ typedef v4u __attribute__((may_alias)) v4u_alias;      // 16-byte reads of memor
 __device__ unsigned long long g_ao_trace[2 * 16 * 12];      // development builds: timestamps of the waves of two workgroups
 #define SBVR_AOSTAMP(i)                                                                                         \
     do {                                                                                                        \
-        if ((blockIdx.x == 0 || blockIdx.x == 100) && (threadIdx.x & 63) == 0)                                  \
-            g_ao_trace[((blockIdx.x != 0) * 16 + (threadIdx.x >> 6)) * 12 + (i)] = wall_clock64();              \
+        if (blockIdx.x == 0 && (blockIdx.y == 0 || blockIdx.y == 12) && (threadIdx.x & 63) == 0)                \
+            g_ao_trace[((blockIdx.y != 0) * 16 + (threadIdx.x >> 6)) * 12 + (i)] = wall_clock64();              \
     } while (0)
 #else
 #define SBVR_AOSTAMP(i) do { } while (0)
@@ -3484,12 +3484,11 @@ sbvr_attn_o_kernel(const AttnOArgs a)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 15, blk = lane >> 4;
-    const int g = static_cast<int>(blockIdx.x) % a.kv_heads;       // key/value head
-    const int e = static_cast<int>(blockIdx.x) / a.kv_heads;       // window of the projection's columns
+    const int g = static_cast<int>(blockIdx.x);        // key/value head (workgroups go to the XCDs by x + 8 y with 8 heads)
+    const int e = static_cast<int>(blockIdx.y);        // window of the projection's columns
     const int N = a.N;
     uint16_t *const kc = a.kcache + static_cast<size_t>(g) * max_seq * kAoHead;
     uint16_t *const vc = a.vcache + static_cast<size_t>(g) * max_seq * kAoHead;
-    const v4u zero4 = {0u, 0u, 0u, 0u};
 
     // -- 1. requests that need no position, in the order they are wanted
     const long long p64 = *a.pos_p;
@@ -3577,14 +3576,13 @@ sbvr_attn_o_kernel(const AttnOArgs a)
     load_line_words<S>(a.cache + static_cast<size_t>(min(lraw, a.L - 1)) * S, cl);
     __builtin_amdgcn_sched_barrier(0);
 
-    // -- 3. scores of the group's four heads (columns 0..3 of the product; the other columns are not used)
+    // -- 3. scores of the group's four heads: columns 0..3 of the product.  (The other twelve columns of B repeat
+    //       them: a column of the product depends on its own column of B only, and theirs are never read.)
     const float scaling = rsqrtf(static_cast<float>(kAoHead));
     v8h qb[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const v4u t = *reinterpret_cast<const v4u_alias *>(qn + (col & (kAoGroup - 1)) * kAoHead + 32 * j + 8 * blk);
-        qb[j] = __builtin_bit_cast(v8h, col < kAoGroup ? t : zero4);
-    }
+    for (int j = 0; j < 4; ++j)
+        qb[j] = __builtin_bit_cast(v8h, v4u(*reinterpret_cast<const v4u_alias *>(qn + (col & (kAoGroup - 1)) * kAoHead + 32 * j + 8 * blk)));
     float mx = -INFINITY;                     // of head `col` over the positions this lane sees
     auto score_block = [&](int tb, v4u (&kw)[4]) __attribute__((always_inline)) {
         if ((p >> 4) == tb) {                 // wave-uniform: the block of the new key, which is not taken from the cache
@@ -3679,8 +3677,7 @@ sbvr_attn_o_kernel(const AttnOArgs a)
             }
         }
         const v4u wb = *reinterpret_cast<const v4u_alias *>(wrow_l + 32 * pb);
-        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, vw),
-                                                   __builtin_bit_cast(v8h, col < kAoGroup ? wb : zero4), o, 0, 0, 0);
+        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, vw), __builtin_bit_cast(v8h, wb), o, 0, 0, 0);
     };
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -3795,7 +3792,7 @@ sbvr_attn_o_kernel(const AttnOArgs a)
 template <int S>
 hipError_t launch_attn_o_inst(const AttnOArgs &a, hipStream_t st)
 {
-    const dim3 grid(static_cast<unsigned>(a.kv_heads * (a.N / kAoCols))), block(kAoThreads);
+    const dim3 grid(static_cast<unsigned>(a.kv_heads), static_cast<unsigned>(a.N / kAoCols)), block(kAoThreads);
     const size_t lds = kAoLdsFixed + 24 * static_cast<size_t>(a.max_seq);
     if (lds > 65536) {          // above what a kernel gets without asking
         static bool raised_on[16] = {};
