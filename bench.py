@@ -150,7 +150,9 @@ def decode_workload(prompt_tokens=128, new_tokens=128):
 def decode_leg(prompt_tokens=128, new_tokens=128):
     """Random-init Llama-3-8B-shaped decoder with SBVR linears (sbvr/decoder.py):
     a 128-token uniform-random prompt, then 128 greedy tokens at batch 1, one
-    HIP-graph replay per token; the figure covers the new tokens only."""
+    HIP-graph replay per prompt token and per 16 new tokens (the same launches
+    either way; the GPU idles some 8 us between two replays); the figure covers
+    the new tokens only."""
     import torch
 
     dec, prompt = decode_workload(prompt_tokens, new_tokens)

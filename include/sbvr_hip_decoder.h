@@ -110,6 +110,18 @@ int sbvr_hip_dec_head_argmax_f16(const void *x, const void *delta, const void *n
                                  int max_seq, const float *cos_table, const float *sin_table, int head_dim,
                                  float *rot_now, void *workspace, void *stream);
 
+/* sbvr_hip_dec_head_argmax_f16 that also starts the next step: x_next[K] <-
+ * embed[*token] for the token it has chosen (embed: (vocab, K) fp16 row-major,
+ * the model's embed_tokens, reference models/sbvr_llama.py:599), so that a
+ * decode step whose input is the previous step's choice needs no launch of
+ * its own for the embedding row.  embed and x_next both NULL: the call above.
+ * Both 16-byte aligned; x_next may be x. */
+int sbvr_hip_dec_head_argmax_embed_f16(const void *x, const void *delta, const void *norm_weight, float eps,
+                                       const void *head, int vocab, int K, void *logits, long long *token,
+                                       long long *generated, long long *pos, int max_seq, const float *cos_table,
+                                       const float *sin_table, int head_dim, float *rot_now, void *workspace,
+                                       const void *embed, void *x_next, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

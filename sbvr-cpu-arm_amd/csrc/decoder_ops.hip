@@ -504,11 +504,11 @@ __global__ void __launch_bounds__(kHeadThreads)
 head_argmax_kernel(const uint16_t *x, const uint16_t *delta, const uint16_t *weight, float eps, const uint16_t *head,
                    int vocab, int rows_per_wave, uint16_t *logits, long long *token, long long *generated, long long *pos,
                    int max_seq, const float *cos_t, const float *sin_t, int half, float *rot_now,
-                   unsigned long long *work)
+                   unsigned long long *work, const uint16_t *embed, uint16_t *x_next)
 {
     constexpr int K = 512 * KI;
     __shared__ unsigned long long best[kHeadThreads / 64];
-    __shared__ long long new_pos;
+    __shared__ long long new_pos, new_token;
     __shared__ int last;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -630,6 +630,7 @@ head_argmax_kernel(const uint16_t *x, const uint16_t *delta, const uint16_t *wei
                 generated[pnow] = bi;
             *pos = pnow + 1;
             new_pos = pnow + 1;
+            new_token = bi;
             __hip_atomic_store(work, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(work + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -642,6 +643,14 @@ head_argmax_kernel(const uint16_t *x, const uint16_t *delta, const uint16_t *wei
             rot_now[d] = cos_t[static_cast<size_t>(row) * half + d];
             rot_now[half + d] = sin_t[static_cast<size_t>(row) * half + d];
         }
+    }
+    // the chosen token's embedding row, where the next step's residual stream starts (every other workgroup has
+    // read x and added its maximum by now, so x_next may be x)
+    if (last && x_next) {
+        const long long t = new_token < 0 ? 0 : (new_token >= vocab ? vocab - 1 : new_token);
+        const v4u_any *src = reinterpret_cast<const v4u_any *>(embed + static_cast<size_t>(t) * K);
+        for (int c = tid; c < K / 8; c += kHeadThreads)
+            reinterpret_cast<v4u_any *>(x_next)[c] = src[c];
     }
 }
 
@@ -731,6 +740,20 @@ int sbvr_hip_dec_head_argmax_f16(const void *x, const void *delta, const void *n
                                  int max_seq, const float *cos_table, const float *sin_table, int head_dim,
                                  float *rot_now, void *workspace, void *stream)
 {
+    return sbvr_hip_dec_head_argmax_embed_f16(x, delta, norm_weight, eps, head, vocab, K, logits, token, generated, pos,
+                                              max_seq, cos_table, sin_table, head_dim, rot_now, workspace, nullptr, nullptr,
+                                              stream);
+}
+
+int sbvr_hip_dec_head_argmax_embed_f16(const void *x, const void *delta, const void *norm_weight, float eps,
+                                       const void *head, int vocab, int K, void *logits, long long *token,
+                                       long long *generated, long long *pos, int max_seq, const float *cos_table,
+                                       const float *sin_table, int head_dim, float *rot_now, void *workspace,
+                                       const void *embed, void *x_next, void *stream)
+{
+    if ((embed == nullptr) != (x_next == nullptr) ||
+        (reinterpret_cast<uintptr_t>(embed) | reinterpret_cast<uintptr_t>(x_next)) % 16)
+        return -1;
     if (!x || !norm_weight || !head || !token || !generated || !pos || !workspace || vocab <= 0 || max_seq <= 0)
         return -1;
     if (rot_now && (!cos_table || !sin_table || head_dim <= 0 || head_dim % 2))
@@ -758,7 +781,8 @@ int sbvr_hip_dec_head_argmax_f16(const void *x, const void *delta, const void *n
                            static_cast<const uint16_t *>(head), vocab, rows_per_wave,                               \
                            static_cast<uint16_t *>(logits), token,                                                  \
                            generated, pos, max_seq, cos_table, sin_table, head_dim / 2, rot_now,                    \
-                           static_cast<unsigned long long *>(workspace));                                           \
+                           static_cast<unsigned long long *>(workspace), static_cast<const uint16_t *>(embed),      \
+                           static_cast<uint16_t *>(x_next));                                                        \
         break
     switch (K) {
         SBVR_HEAD(1); SBVR_HEAD(2); SBVR_HEAD(4); SBVR_HEAD(8); SBVR_HEAD(16);

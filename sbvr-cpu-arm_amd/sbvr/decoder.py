@@ -10,8 +10,9 @@ weight gives.  Embedding and output head stay fp16, as in the reference's
 model.  Everything else (norms, rotary embedding, attention over the cache) is
 a handful of small kernels in this package's library or plain torch ops.
 
-One decode step is recorded into a HIP graph once and replayed per token; the
-token id and the position live on the device, so a replay needs no host work.
+One decode step is recorded into a HIP graph once and replayed per token (and
+sixteen steps into a second graph, replayed per sixteen new tokens); the token
+id and the position live on the device, so a replay needs no host work.
 """
 import time
 from dataclasses import dataclass
@@ -123,6 +124,7 @@ class SbvrLlamaDecoder:
         self.logits = torch.empty((1, s.vocab), dtype=torch.float16, device=dev)
         self.head_ws = torch.zeros(2, dtype=torch.int64, device=dev)              # cross-workgroup argmax of the head kernel
         self.graph = None
+        self.graph_many, self.steps_per_replay = None, 1
         self.stream = torch.cuda.Stream(device=dev)
         # probe(layer, residual): called by an eager fused step with the residual stream as it enters each layer
         # (layer 0: the embedding row) and, as layer == layers, as it enters the final norm; for tests
@@ -137,9 +139,10 @@ class SbvrLlamaDecoder:
         return self.encoded_bytes() + self.lm_head.numel() * 2 + self.shape.hidden * 2
 
     # -- one token -------------------------------------------------------------
-    def step(self):
-        """One decode step."""
-        return self._step_fused() if self.fused else self._step_unfused()
+    def step(self, gather=True):
+        """One decode step.  gather=False (fused steps with the one-launch end of the step): the input row is
+        not looked up, it is what the previous step's last launch left for the token it chose."""
+        return self._step_fused(gather) if self.fused else self._step_unfused()
 
     def _step_unfused(self):
         """8 launches per layer (norm, q|k|v, attention, o, norm, gate|up,
@@ -162,7 +165,7 @@ class SbvrLlamaDecoder:
         hip.dec_argmax_advance(logits, self.tok, self.generated, self.pos, self.cos, self.sin, self.rot_now)
         return logits
 
-    def _step_fused(self):
+    def _step_fused(self, gather=True):
         """One launch for the end of the step (final norm, head, argmax) where the
         hidden size has a kernel, and 5 launches per layer: q|k|v (with the residual add and norm in front),
         attention, o, gate|up (same), down (with SiLU*up in front); 4 with attention and o in one launch
@@ -171,7 +174,8 @@ class SbvrLlamaDecoder:
         sum to the other, since its workgroups do not run in step."""
         s = self.shape
         a, b, ctx = self.x, self.x_alt, self.ctx
-        torch.index_select(self.embed, 0, self.tok, out=a)            # (1, hidden)
+        if gather or not hip.dec_head_argmax_supported(s.hidden):
+            torch.index_select(self.embed, 0, self.tok, out=a)        # (1, hidden)
         delta = self.zero
         for number, layer in enumerate(self.layers):
             qkv = layer["qkv"].after_add_rmsnorm(a, delta, layer["norm1"], s.rms_eps, b)
@@ -191,9 +195,11 @@ class SbvrLlamaDecoder:
         if self.probe is not None:
             self.probe(len(self.layers), (a.float() + delta.float()).to(torch.float16))
         if hip.dec_head_argmax_supported(s.hidden):
-            # final norm, head, argmax and position advance in one launch
+            # final norm, head, argmax and position advance in one launch, which also leaves the chosen token's
+            # embedding row where the next step starts
             hip.dec_head_argmax(a, delta, self.final_norm, s.rms_eps, self.lm_head, self.logits, self.tok,
-                                self.generated, self.pos, self.head_ws, self.cos, self.sin, self.rot_now)
+                                self.generated, self.pos, self.head_ws, self.cos, self.sin, self.rot_now,
+                                embed=self.embed, x_next=a)
             return self.logits
         hip.dec_add_rmsnorm(a, delta, self.final_norm, self.h, s.rms_eps)
         logits = torch.matmul(self.h, self.lm_head.t())                 # (1, vocab)
@@ -201,9 +207,12 @@ class SbvrLlamaDecoder:
         return logits
 
     # -- driving ---------------------------------------------------------------
-    def capture(self):
+    def capture(self, steps_per_replay=16):
         """Records one step into a HIP graph (after one eager step on the same
-        stream, which also creates the operator's workspace for that stream)."""
+        stream, which also creates the operator's workspace for that stream), and
+        `steps_per_replay` steps into a second one: token and position live on the
+        device, so consecutive steps are the same launches, and between two replays
+        the GPU idles for some 8 us that a replay of several steps pays once."""
         with torch.cuda.stream(self.stream):
             self.step()
             torch.cuda.synchronize()
@@ -211,6 +220,13 @@ class SbvrLlamaDecoder:
             with torch.cuda.graph(self.graph, stream=self.stream):
                 self.step()
             torch.cuda.synchronize()
+            self.graph_many, self.steps_per_replay = None, int(steps_per_replay)
+            if self.steps_per_replay > 1:
+                self.graph_many = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(self.graph_many, stream=self.stream):
+                    for _ in range(self.steps_per_replay):
+                        self.step(gather=False)     # (each step's input is the choice of the step before)
+                torch.cuda.synchronize()
         self.reset()
 
     def reset(self):
@@ -242,7 +258,12 @@ class SbvrLlamaDecoder:
                 self._advance()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            for _ in range(new_tokens):
+            left = new_tokens
+            many = self.graph_many if self.graph is not None else None
+            while many is not None and left >= self.steps_per_replay:
+                many.replay()
+                left -= self.steps_per_replay
+            for _ in range(left):
                 self._advance()
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0

@@ -75,6 +75,8 @@ def _load():
     lib.sbvr_hip_dec_argmax_advance_f16.argtypes = [vp, i, vp, vp, vp, i, vp, vp, i, vp, vp]
     lib.sbvr_hip_dec_head_argmax_f16.argtypes = [vp, vp, vp, ctypes.c_float, vp, i, i, vp, vp, vp, vp, i, vp, vp, i,
                                                  vp, vp, vp]
+    lib.sbvr_hip_dec_head_argmax_embed_f16.argtypes = [vp, vp, vp, ctypes.c_float, vp, i, i, vp, vp, vp, vp, i, vp, vp, i,
+                                                       vp, vp, vp, vp, vp]
     lib.sbvr_hip_encoder_group_mse_f16.argtypes = [vp, vp, vp, i, i, i, i, vp]
     lib.sbvr_hip_online_encode_f16.argtypes = [vp, vp, vp, i, i, i, i, vp]
     _lib = lib
@@ -495,9 +497,11 @@ def dec_head_argmax_supported(hidden):
 
 
 def dec_head_argmax(x, delta, weight, eps, head, logits, token, generated, pos, workspace, cos=None, sin=None,
-                    rot_now=None):
+                    rot_now=None, embed=None, x_next=None):
     """Final residual add + RMSNorm, fp16 output head, argmax and position advance in one launch.
-    ``head`` (vocab, hidden) fp16; ``logits`` (vocab,) fp16 or None; ``workspace``: two int64 zeros."""
+    ``head`` (vocab, hidden) fp16; ``logits`` (vocab,) fp16 or None; ``workspace``: two int64 zeros.
+    ``embed`` (vocab, hidden) fp16 and ``x_next`` (hidden): the chosen token's embedding row is left in ``x_next``
+    (which may be ``x``) for the next step."""
     for t, name in ((x, "x"), (weight, "weight"), (head, "head")) + (((delta, "delta"),) if delta is not None else ()) \
             + (((logits, "logits"),) if logits is not None else ()):
         _want(t, name, torch.float16)
@@ -514,12 +518,21 @@ def dec_head_argmax(x, delta, weight, eps, head, logits, token, generated, pos, 
         head_dim = rot_now.numel()
         if cos.shape != (generated.numel(), head_dim // 2) or sin.shape != cos.shape:
             raise SbvrHipError("dec_head_argmax: rotary tables must be (max_seq, head_dim / 2)")
-    _dec_check(_load().sbvr_hip_dec_head_argmax_f16(
+    if (embed is None) != (x_next is None):
+        raise SbvrHipError("dec_head_argmax: embed and x_next go together")
+    if embed is not None:
+        _want(embed, "embed", torch.float16, 2)
+        _want(x_next, "x_next", torch.float16)
+        if tuple(embed.shape) != (vocab, hidden) or x_next.numel() != hidden:
+            raise SbvrHipError("dec_head_argmax: embed must be (vocab, hidden) and x_next hold hidden elements")
+    _dec_check(_load().sbvr_hip_dec_head_argmax_embed_f16(
         x.data_ptr(), delta.data_ptr() if delta is not None else None, weight.data_ptr(), float(eps), head.data_ptr(),
         vocab, hidden, logits.data_ptr() if logits is not None else None, token.data_ptr(), generated.data_ptr(),
         pos.data_ptr(), generated.numel(), cos.data_ptr() if rot_now is not None else None,
         sin.data_ptr() if rot_now is not None else None, head_dim,
-        rot_now.data_ptr() if rot_now is not None else None, workspace.data_ptr(), _stream()), "head_argmax")
+        rot_now.data_ptr() if rot_now is not None else None, workspace.data_ptr(),
+        embed.data_ptr() if embed is not None else None, x_next.data_ptr() if embed is not None else None, _stream()),
+        "head_argmax")
     return logits
 
 

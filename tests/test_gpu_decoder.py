@@ -305,6 +305,16 @@ def test_head_argmax_kernel(hidden, vocab, with_delta):
         assert int(ws[0]) == 0 and int(ws[1]) == 0
     # the input row is left alone
     assert torch.equal(xd.cpu(), x)
+    # the form that also leaves the chosen token's embedding row for the next step, in another buffer and in x itself
+    embed = torch.randn((vocab, hidden), generator=gen).to(torch.float16).to(dev)
+    x_next = torch.zeros(hidden, dtype=torch.float16, device=dev)
+    first = int(tok)
+    hip.dec_head_argmax(xd, dd, wd, 1e-5, hd, logits, tok, generated, pos, ws, cos, sin, rot, embed=embed, x_next=x_next)
+    torch.cuda.synchronize()
+    assert int(tok) == first and torch.equal(x_next, embed[first]) and torch.equal(xd.cpu(), x)
+    hip.dec_head_argmax(xd, dd, wd, 1e-5, hd, logits, tok, generated, pos, ws, cos, sin, rot, embed=embed, x_next=xd)
+    torch.cuda.synchronize()
+    assert int(tok) == first and torch.equal(xd, embed[first]) and int(ws[0]) == 0 and int(ws[1]) == 0
 
 
 def test_head_argmax_tie_and_nan():
