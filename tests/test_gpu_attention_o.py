@@ -145,6 +145,32 @@ def test_formats_and_shapes(oracle, kw):
     _run_case(oracle, 256, 77, ready_rotation=True, seed=3, **kw)
 
 
+@pytest.mark.parametrize("stored,used", [(-3, 0), (64 + 5, 63)])
+def test_position_outside_the_cache_is_clamped(stored, used):
+    """*pos below 0 or beyond the cache is taken as the nearest valid position, as by the two-launch kernel."""
+    from sbvr import hip
+    dev = torch.device("cuda:0")
+    heads, kv_heads, hd, max_seq, N, S, G, L = 32, 8, HEAD_DIM, 64, 4096, 4, 128, 256
+    bvr, idx, cache = (t.to(dev) for t in _encoding(N, heads * hd, S, G, L, 21))
+    gen = torch.Generator().manual_seed(stored + 100)
+    qkv = torch.randn((1, (heads + 2 * kv_heads) * hd), generator=gen).to(torch.float16).to(dev)
+    ang = torch.rand((max_seq, hd // 2), generator=gen, dtype=torch.float64) * 6.28
+    cos, sin = torch.cos(ang).float().to(dev), torch.sin(ang).float().to(dev)
+    kc = torch.randn((kv_heads, max_seq, hd), generator=gen).to(torch.float16).to(dev)
+    vc = torch.randn((kv_heads, max_seq, hd), generator=gen).to(torch.float16).to(dev)
+    results = []
+    for p in (stored, used):
+        k2, v2 = hip.attention_o_cache_layout(kc), hip.attention_o_cache_layout(vc, values=True)
+        ctx = torch.zeros((1, heads * hd), dtype=torch.float16, device=dev)
+        out = torch.empty((1, N), dtype=torch.float16, device=dev)
+        hip.dec_attention_o(qkv, cos, sin, torch.tensor([p], device=dev), k2, v2, heads, kv_heads, hd, bvr, idx, cache, None, G,
+                            out=out, ctx=ctx)
+        torch.cuda.synchronize()
+        results.append((out.clone(), ctx.clone(), k2, v2))
+    for a, b in zip(results[0], results[1]):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
 def test_refusals():
     """Shapes the launch does not take are refused, and so is a call without its accumulators."""
     import ctypes
